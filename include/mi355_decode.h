@@ -945,25 +945,32 @@ int32_t mi355_latent_window_attn(void* out, int64_t out_stride, int64_t out_head
 
 /*
  * Mixture-of-experts feed-forward.  A routed row is (token t, choice k), number t * top + k.
- *   moe_route         from fp32 router logits [tokens, experts]: score = sigmoid(logit); experts are
- *                     chosen by score + correction among the experts of the `keep` best of `groups`
- *                     groups of neighbouring experts (a group scores the sum of its two largest
- *                     score + correction); ids [tokens, top], weights [tokens, top] = the chosen
- *                     experts' scores (no correction, not renormalised)
+ *   moe_route         from fp32 router logits (rows of logits_stride floats, the first `experts` of
+ *                     them router outputs): score = sigmoid(logit), or with `softmax` a softmax over
+ *                     the router outputs; experts are chosen by score + correction among the experts
+ *                     of the `keep` best of `groups` groups of neighbouring experts (a group scores
+ *                     the sum of its two largest score + correction, or with `group_max` the
+ *                     largest); ids [tokens, top], weights [tokens, top] = the chosen experts'
+ *                     scores times weight_scale (no correction, not renormalised)
  *   moe_sort          routed rows by expert: offsets [experts + 1], perm[position] = row,
  *                     inv[row] = position
  *   moe_gather_rows   xs[position] = x[perm[position] / top] for num_rows positions (pad_to 0); with
  *                     pad_to > 0, num_rows = experts * pad_to and xs[e * pad_to + j] is the j-th row of
  *                     expert e, zeros past its count (one batched product over all experts then)
- *   moe_gate_up_rows  act[position] = silu(Wg[e] x[t]) * (Wu[e] x[t]); w_gate_up [experts, 2 ff, width]
+ *   moe_gate_up_rows  act[position] = a(Wg[e] x[t], Wu[e] x[t]); w_gate_up [experts, 2 ff, width];
+ *                     a(g, u) = silu(g) * u (act 0), or with g = min(g, limit), u = clamp(u, -limit,
+ *                     limit): g * sigmoid(1.702 g) * (u + 1) (act 1)
  *   moe_down_rows     y[position] = Wd[e] act[position]; w_down [experts, width, ff]
- *   moe_silu_and_mul  out = silu(x[:, :ff]) * x[:, ff:]
+ *   moe_silu_and_mul  out = a(x[:, :ff], x[:, ff:])
  *   moe_combine       out[t] = sum_k weights[t, k] * y[inv[t * top + k]]; with pad_to > 0, y holds every
- *                     expert's rows padded to pad_to (ids and offsets locate them)
+ *                     expert's rows padded to pad_to (ids and offsets locate them).  x not null: a
+ *                     chosen id >= num_real is an identity expert, its row is x[t].  shared not null:
+ *                     + shared[t] * sigmoid(shared_gate[t * shared_gate_stride]) (gate null: + shared[t])
  */
-int32_t mi355_moe_route(int32_t* ids, float* weights, const float* logits, const float* correction,
-                        int64_t num_tokens, int32_t experts, int32_t top, int32_t groups, int32_t keep,
-                        void* stream);
+int32_t mi355_moe_route(int32_t* ids, float* weights, const float* logits, int64_t logits_stride,
+                        const float* correction, int64_t num_tokens, int32_t experts, int32_t top,
+                        int32_t groups, int32_t keep, int32_t softmax, int32_t group_max,
+                        float weight_scale, void* stream);
 int32_t mi355_moe_sort(int32_t* offsets, int32_t* perm, int32_t* inv, const int32_t* ids,
                        int64_t num_rows, int32_t experts, void* stream);
 int32_t mi355_moe_gather_rows(void* xs, const void* x, const int32_t* perm, const int32_t* offsets,
@@ -971,14 +978,68 @@ int32_t mi355_moe_gather_rows(void* xs, const void* x, const int32_t* perm, cons
                               int32_t dtype, void* stream);
 int32_t mi355_moe_gate_up_rows(void* act, const void* x, const void* w_gate_up, const int32_t* offsets,
                                const int32_t* perm, int32_t experts, int32_t top, int32_t width,
-                               int32_t ff, int32_t dtype, void* stream);
+                               int32_t ff, int32_t act_fn, float limit, int32_t dtype, void* stream);
 int32_t mi355_moe_down_rows(void* y, const void* act, const void* w_down, const int32_t* offsets,
                             int32_t experts, int32_t width, int32_t ff, int32_t dtype, void* stream);
-int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_rows, int32_t ff, int32_t dtype,
-                               void* stream);
+int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_rows, int32_t ff, int32_t act_fn,
+                               float limit, int32_t dtype, void* stream);
 int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const float* weights,
                           const int32_t* ids, const int32_t* offsets, int32_t pad_to,
-                          int64_t num_tokens, int32_t top, int32_t width, int32_t dtype, void* stream);
+                          int64_t num_tokens, int32_t top, int32_t width, const void* x,
+                          int32_t num_real, const void* shared, const float* shared_gate,
+                          int64_t shared_gate_stride, int32_t dtype, void* stream);
+
+/*
+ * A decoder with a hashed previous-token embedding, sinusoidal positions, softmax attention inside
+ * blocks of positions with a logarithmic distance penalty, and a per-channel gated recurrence.
+ *   embed_bigram_pos_f32  out[t] = embed[id] + bigram[(prev * mul_prev + id * mul_cur) % buckets]
+ *                         (row `buckets` at position 0) + sinusoid: entry 2i = sin(p * freq[i]), entry
+ *                         2i + 1 = cos; the previous token of a chunk's first row is prev_tokens[slot].
+ *                         bigram / freq may be null (none)
+ *   prev_token_update     prev_tokens[slot of chunk s] = the chunk's last token (after the embedding)
+ *   relu_squared          out = max(x, 0)^2
+ *   qk_norm_kv_write      q <- rms(q) * q_weight per head, in place; K pages <- rms(k) * k_weight per
+ *                         head; V pages <- v (rows of the caller's choice).  Weights fp32 [head_dim]
+ *   softmax_bias_attn     out[t,h] = sigmoid(gate) * sum_j softmax_j(q.k_j * scale - r1[h] ln(1 + r2[h]
+ *                         (p - j))) v_j over the keys j <= p with j >= (p / block) * block (block 0: all)
+ *                         and, window > 0, j > p - window.  gate: one number per head or
+ *                         (gate_per_channel) per output channel; r1 / r2 null: no penalty.  tiles as for
+ *                         sigmoid_window_attn; workspace (softmax_bias_attn_workspace floats) with
+ *                         num_splits > 1 spreads a tile's keys over that many workgroups
+ *   mingru_scan           S <- (1 - z) S + z c per channel, z = sigmoid(zp + z_bias), u = xp + x_bias,
+ *                         c = u + 1/2 (u >= 0) or sigmoid(u); out = S * silu(gp); zp / xp / gp are the
+ *                         column ranges z_off / x_off / g_off of the projection rows; state fp32
+ *                         [slots, channels], reset by a chunk that starts at position 0
+ */
+int32_t mi355_embed_bigram_pos_f32(float* out, const void* embed, const void* bigram, const int64_t* ids,
+                                   const int64_t* positions, const int32_t* cu_seqlens,
+                                   const int32_t* tok_seq, const int32_t* state_slots,
+                                   const int32_t* prev_tokens, const float* freq, int64_t num_tokens,
+                                   int32_t width, int64_t vocab, int64_t buckets, int64_t mul_prev,
+                                   int64_t mul_cur, int32_t dtype, void* stream);
+int32_t mi355_prev_token_update(int32_t* prev_tokens, const int64_t* ids, const int32_t* cu_seqlens,
+                                const int32_t* state_slots, int32_t num_seqs, void* stream);
+int32_t mi355_relu_squared(void* out, const void* x, int64_t numel, int32_t dtype, void* stream);
+int32_t mi355_qk_norm_kv_write(void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                               int64_t v_stride, const float* q_weight, const float* k_weight,
+                               const int64_t* slot_mapping, void* k_cache, void* v_cache,
+                               int64_t num_tokens, int32_t num_heads, int32_t num_kv_heads,
+                               int32_t head_dim, int32_t v_dim, float eps, int32_t dtype, void* stream);
+int64_t mi355_softmax_bias_attn_workspace(int64_t num_tokens, int32_t num_heads, int32_t v_dim,
+                                          int32_t num_splits);
+int32_t mi355_softmax_bias_attn(void* out, const void* q, int64_t q_stride, const void* k_cache,
+                                const void* v_cache, const int32_t* block_tables, int32_t max_blocks,
+                                const int32_t* tok_seq, const int64_t* positions, const float* r1,
+                                const float* r2, const void* gate, int64_t gate_stride,
+                                int32_t gate_per_channel, int64_t num_tokens, int32_t num_heads,
+                                int32_t num_kv_heads, int32_t head_dim, int32_t v_dim, int32_t block,
+                                int32_t window, float scale, const int32_t* tiles, int32_t num_tiles,
+                                float* workspace, int32_t num_splits, int32_t dtype, void* stream);
+int32_t mi355_mingru_scan(void* out, const void* proj, int64_t stride, int32_t z_off, int32_t x_off,
+                          int32_t g_off, const float* z_bias, const float* x_bias, float* state,
+                          const int32_t* cu_seqlens, const int64_t* positions,
+                          const int32_t* state_slots, int32_t num_seqs, int64_t num_tokens,
+                          int32_t channels, int32_t long_chunks, int32_t dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,8 +1,9 @@
 // Mixture-of-experts feed-forward: routing, the expert-sorted row order, and the expert products for
 // steps of few rows.
-//   moe_route           sigmoid scores from fp32 router logits; experts are picked by score + correction
-//                       among the experts of the best `keep` of `count` groups of neighbours (a group
-//                       scores the sum of its two best), and weighted by the score without correction
+//   moe_route           scores from fp32 router logits (a sigmoid each, or a softmax over all of them);
+//                       experts are picked by score + correction among the experts of the best `keep` of
+//                       `count` groups of neighbours (a group scores the sum of its two best, or its
+//                       best), and weighted by the score without correction, times a constant
 //   moe_sort            rows (token, choice) ordered by expert: offsets[E + 1], perm[position] = row,
 //                       inv[row] = position
 //   moe_gather_rows     xs[position] = x[perm[position] / top]; or every expert's rows padded to a common count
@@ -11,7 +12,11 @@
 //   moe_down_rows       y[position] = Wd[e] a[position], the same way; both on the matrix cores where the
 //                       sizes allow (16-bit storage, widths multiples of 32 / 16)
 //   moe_silu_and_mul    a = silu(gu[:, :F]) * gu[:, F:] (any storage type)
-//   moe_combine         out[t] = sum_k weight[t, k] * y[inv[t * top + k]]
+//   moe_combine         out[t] = sum_k weight[t, k] * y[inv[t * top + k]]; a chosen id at or past `num_real`
+//                       is an identity expert and stands for x[t]; a shared expert's rows join, times the
+//                       sigmoid of one fp32 number per token
+// The gated activation of an expert is silu(g) * u, or (act 1) with g = min(g, limit) and
+// u = clamp(u, -limit, limit): g * sigmoid(1.702 g) * (u + 1).
 // Routing, scores and the weighted sum are fp32; activations and expert weights are stored in the
 // dtype argument's type, products accumulate in fp32.
 #include "common.h"
@@ -22,16 +27,25 @@ constexpr int kMaxGroups = 64;
 constexpr int kMaxTop = 16;
 
 __global__ __launch_bounds__(64) void moe_route_kernel(int32_t* __restrict__ ids, float* __restrict__ wts,
-                                                       const float* __restrict__ z, const float* __restrict__ corr,
-                                                       int64_t T, int E, int top, int count, int keep) {
+                                                       const float* __restrict__ z, int64_t z_stride,
+                                                       const float* __restrict__ corr, int64_t T, int E, int top, int count,
+                                                       int keep, int softmax, int group_max, float wscale) {
   const int64_t t = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x;
   if (t >= T) return;
-  const float* zr = z + t * E;
+  const float* zr = z + t * z_stride;
   const int per = E / count;
   const float ninf = -__builtin_inff();
-  auto choice = [&](int e) {
-    return 1.0f / (1.0f + expf(-MI355_LD(float, z, zr + e))) + MI355_LD(float, corr, corr + e);
+  float zmax = ninf, zsum = 1.0f;
+  if (softmax) {
+    for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, MI355_LD(float, z, zr + e));
+    zsum = 0.f;
+    for (int e = 0; e < E; ++e) zsum += expf(MI355_LD(float, z, zr + e) - zmax);
+  }
+  auto score = [&](int e) {
+    const float v = MI355_LD(float, z, zr + e);
+    return softmax ? expf(v - zmax) / zsum : 1.0f / (1.0f + expf(-v));
   };
+  auto choice = [&](int e) { return score(e) + MI355_LD(float, corr, corr + e); };
   // the groups that stay: `keep` rounds of picking the best group not yet picked
   uint64_t allowed = 0;
   if (keep >= count) {
@@ -47,7 +61,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int32_t* __restrict__ ids
           const float c = choice(g * per + i);
           if (c > a) { b = a; a = c; } else if (c > b) { b = c; }
         }
-        const float gs = per > 1 ? a + b : a;
+        const float gs = (per > 1 && !group_max) ? a + b : a;
         if (best < 0 || gs > bs) { best = g; bs = gs; }
       }
       allowed |= 1ull << best;
@@ -67,7 +81,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int32_t* __restrict__ ids
     }
     picked[r] = best;
     MI355_ST(int32_t, ids, ids + t * top + r, best);
-    MI355_ST(float, wts, wts + t * top + r, 1.0f / (1.0f + expf(-MI355_LD(float, z, zr + best))));
+    MI355_ST(float, wts, wts + t * top + r, score(best) * wscale);
   }
 }
 
@@ -85,21 +99,39 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 // lanes from the choice scores in LDS; every pick is a maximum over the wave.
 template <int EPL>
 __global__ __launch_bounds__(256) void moe_route_wave_kernel(int32_t* __restrict__ ids, float* __restrict__ wts,
-                                                             const float* __restrict__ z, const float* __restrict__ corr,
-                                                             int64_t T, int E, int top, int count, int keep) {
+                                                             const float* __restrict__ z, int64_t z_stride,
+                                                             const float* __restrict__ corr, int64_t T, int E, int top,
+                                                             int count, int keep, int softmax, int group_max, float wscale) {
   __shared__ float ch[4][64 * EPL];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   int64_t t = blockIdx.x * 4 + wave;
   const bool live = t < T;
   if (!live) t = T - 1;                                 // (every wave reaches the barrier; nothing stored)
-  const float* zr = z + t * E;
+  const float* zr = z + t * z_stride;
   const float ninf = -__builtin_inff();
   const int per = E / count;
+  float zmax = ninf, zsum = 1.0f;
+  if (softmax) {                                        // over all router outputs, in fp32
+#pragma unroll
+    for (int i = 0; i < EPL; ++i)
+      if (lane + 64 * i < E) zmax = fmaxf(zmax, MI355_LD(float, z, zr + lane + 64 * i));
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) zmax = fmaxf(zmax, __shfl_xor(zmax, off, 64));
+    float part = 0.f;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i)
+      if (lane + 64 * i < E) part += expf(MI355_LD(float, z, zr + lane + 64 * i) - zmax);
+    zsum = wave_sum(part);
+  }
+  auto score = [&](int e) {
+    const float v = MI355_LD(float, z, zr + e);
+    return softmax ? expf(v - zmax) / zsum : 1.0f / (1.0f + expf(-v));
+  };
   float c[EPL];
 #pragma unroll
   for (int i = 0; i < EPL; ++i) {
     const int e = lane + 64 * i;
-    c[i] = e < E ? 1.0f / (1.0f + expf(-MI355_LD(float, z, zr + e))) + MI355_LD(float, corr, corr + e) : ninf;
+    c[i] = e < E ? score(e) + MI355_LD(float, corr, corr + e) : ninf;
     if (c[i] != c[i]) c[i] = -3.0e38f;                  // a NaN logit ranks last but stays a valid pick: ids are indices downstream
     ch[wave][e] = c[i];
   }
@@ -112,7 +144,7 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(int32_t* __restrict
         const float v = ch[wave][lane * per + i];
         if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
       }
-      gs = per > 1 ? a + b : a;
+      gs = (per > 1 && !group_max) ? a + b : a;
     }
     uint64_t allowed = 0;
     bool mine = false;                                  // this lane's group has been picked
@@ -143,7 +175,7 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(int32_t* __restrict
       if (lane + 64 * i == e) c[i] = ninf;              // taken
     if (live && lane == 0) {
       MI355_ST(int32_t, ids, ids + t * top + r, e);
-      MI355_ST(float, wts, wts + t * top + r, 1.0f / (1.0f + expf(-MI355_LD(float, z, zr + e))));
+      MI355_ST(float, wts, wts + t * top + r, score(e) * wscale);
     }
   }
 }
@@ -202,6 +234,14 @@ __global__ __launch_bounds__(256) void moe_gather_rows_kernel(typename Elem<T>::
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
+// the gated activation of an expert (see the head of this file)
+__device__ __forceinline__ float gated_act(float g, float u, int act, float limit) {
+  if (act == 0) return silu_f(g) * u;
+  g = fminf(g, limit);
+  u = fminf(fmaxf(u, -limit), limit);
+  return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+}
+
 // Rows of an expert are taken kRowBlock at a time, so that a weight element is loaded once per block
 // of rows and not once per row.
 constexpr int kRowBlock = 8;
@@ -257,7 +297,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_rows_kernel(typename Elem<T>:
                                                                const typename Elem<T>::S* __restrict__ x,
                                                                const typename Elem<T>::S* __restrict__ w_gate_up,
                                                                const int32_t* __restrict__ offsets,
-                                                               const int32_t* __restrict__ perm, int top, int W, int F) {
+                                                               const int32_t* __restrict__ perm, int top, int W, int F,
+                                                               int act, float limit) {
   typedef typename Elem<T>::S E;
   const int e = blockIdx.y, lane = threadIdx.x & 63;
   const int f = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -279,7 +320,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_rows_kernel(typename Elem<T>:
     for (int r = 0; r < kRowBlock; ++r) {
       if (lane == r && p0 + r < hi) {
         const float gr = elem_to_f<T>(elem_from_f<T>(g[r])), ur = elem_to_f<T>(elem_from_f<T>(u[r]));   // as stored by a product
-        MI355_STF(T, a, a + static_cast<int64_t>(p0 + r) * F + f, silu_f(gr) * ur);
+        MI355_STF(T, a, a + static_cast<int64_t>(p0 + r) * F + f, gated_act(gr, ur, act, limit));
       }
     }
   }
@@ -316,7 +357,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(uint16_t* __restrict__ a, const uint16_t* __restrict__ x,
                                                                const uint16_t* __restrict__ w_gate_up,
                                                                const int32_t* __restrict__ offsets,
-                                                               const int32_t* __restrict__ perm, int top, int W, int F) {
+                                                               const int32_t* __restrict__ perm, int top, int W, int F,
+                                                               int act, float limit) {
   const int e = blockIdx.y, lane = threadIdx.x & 63, li = lane & 15, kk = lane >> 4;
   const int f0 = (blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 16;
   if (f0 >= F) return;
@@ -335,7 +377,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_mfma_kernel(uint16_t* __restr
     if (p0 + li < hi) {
       float out[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) out[r] = silu_f(round_f<T>(g[r])) * round_f<T>(u[r]);      // as stored by a product
+      for (int r = 0; r < 4; ++r) out[r] = gated_act(round_f<T>(g[r]), round_f<T>(u[r]), act, limit);      // as stored by a product
       MI355_ST(uint2, a, a + static_cast<int64_t>(p0 + li) * F + f0 + 4 * kk,
                make_uint2(T::pack2(out[0], out[1]), T::pack2(out[2], out[3])));
     }
@@ -369,13 +411,13 @@ __global__ __launch_bounds__(256) void moe_down_mfma_kernel(uint16_t* __restrict
 template <typename T>
 __global__ __launch_bounds__(256) void moe_silu_and_mul_kernel(typename Elem<T>::S* __restrict__ out,
                                                                const typename Elem<T>::S* __restrict__ x, int64_t rows,
-                                                               int F) {
+                                                               int F, int act, float limit) {
   const int64_t total = rows * F;
   for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
     const int64_t r = i / F;
     const int f = static_cast<int>(i % F);
-    MI355_STF(T, out, out + i, silu_f(MI355_LDF(T, x, x + r * 2 * F + f)) * MI355_LDF(T, x, x + r * 2 * F + F + f));
+    MI355_STF(T, out, out + i, gated_act(MI355_LDF(T, x, x + r * 2 * F + f), MI355_LDF(T, x, x + r * 2 * F + F + f), act, limit));
   }
 }
 
@@ -384,18 +426,28 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(typename Elem<T>::S* _
                                                           const typename Elem<T>::S* __restrict__ y,
                                                           const int32_t* __restrict__ inv, const float* __restrict__ wts,
                                                           const int32_t* __restrict__ ids,
-                                                          const int32_t* __restrict__ offsets, int cap, int top, int W) {
+                                                          const int32_t* __restrict__ offsets, int cap, int top, int W,
+                                                          const typename Elem<T>::S* __restrict__ x, int num_real,
+                                                          const typename Elem<T>::S* __restrict__ shared,
+                                                          const float* __restrict__ shared_gate, int64_t shared_gate_stride) {
   const int64_t t = blockIdx.x;
+  float sg = 0.f;
+  if (shared != nullptr)
+    sg = shared_gate != nullptr ? 1.0f / (1.0f + expf(-MI355_LD(float, shared_gate, shared_gate + t * shared_gate_stride))) : 1.0f;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float s = 0.f;
     for (int k = 0; k < top; ++k) {
-      int64_t p = MI355_LD(int32_t, inv, inv + t * top + k);
-      if (cap > 0) {                                    // y holds every expert's rows padded to cap
-        const int e = MI355_LD(int32_t, ids, ids + t * top + k);
-        p += static_cast<int64_t>(e) * cap - MI355_LD(int32_t, offsets, offsets + e);
+      const int e = ids != nullptr ? MI355_LD(int32_t, ids, ids + t * top + k) : 0;
+      const float w = MI355_LD(float, wts, wts + t * top + k);
+      if (x != nullptr && e >= num_real) {              // an identity expert: the input itself
+        s += w * MI355_LDF(T, x, x + t * W + c);
+        continue;
       }
-      s += MI355_LD(float, wts, wts + t * top + k) * MI355_LDF(T, y, y + p * W + c);
+      int64_t p = MI355_LD(int32_t, inv, inv + t * top + k);
+      if (cap > 0) p += static_cast<int64_t>(e) * cap - MI355_LD(int32_t, offsets, offsets + e);   // y: every expert's rows padded to cap
+      s += w * MI355_LDF(T, y, y + p * W + c);
     }
+    if (shared != nullptr) s += sg * MI355_LDF(T, shared, shared + t * W + c);
     MI355_STF(T, out, out + t * W + c, s);
   }
 }
@@ -406,10 +458,12 @@ using namespace mi355;
 
 #define REQ_DTYPE(dtype) MI355_REQUIRE((dtype) >= MI355_BF16 && (dtype) <= MI355_F32, MI355_ERR_UNSUPPORTED, "dtype code %d", (dtype))
 
-extern "C" int32_t mi355_moe_route(int32_t* ids, float* weights, const float* logits, const float* correction,
-                                   int64_t num_tokens, int32_t experts, int32_t top, int32_t groups, int32_t keep,
+extern "C" int32_t mi355_moe_route(int32_t* ids, float* weights, const float* logits, int64_t logits_stride,
+                                   const float* correction, int64_t num_tokens, int32_t experts, int32_t top,
+                                   int32_t groups, int32_t keep, int32_t softmax, int32_t group_max, float weight_scale,
                                    void* stream) {
   MI355_REQUIRE(ids && weights && logits && correction, MI355_ERR_INVALID, "moe_route: null pointer");
+  MI355_REQUIRE(logits_stride >= experts, MI355_ERR_INVALID, "moe_route: logit rows shorter than the experts");
   MI355_REQUIRE(num_tokens >= 0 && experts > 0 && top > 0 && groups > 0 && keep > 0 && keep <= groups &&
                     experts % groups == 0,
                 MI355_ERR_INVALID, "moe_route: %d experts in %d groups, %d kept, %d chosen", experts, groups, keep, top);
@@ -421,15 +475,16 @@ extern "C" int32_t mi355_moe_route(int32_t* ids, float* weights, const float* lo
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 wgrid(static_cast<unsigned>((num_tokens + 3) / 4));
 #define MI355_ROUTE(EPL)                                                                                            \
-  hipLaunchKernelGGL((moe_route_wave_kernel<EPL>), wgrid, dim3(256), 0, s, ids, weights, logits, correction,        \
-                     num_tokens, experts, top, groups, keep)
+  hipLaunchKernelGGL((moe_route_wave_kernel<EPL>), wgrid, dim3(256), 0, s, ids, weights, logits, logits_stride,     \
+                     correction, num_tokens, experts, top, groups, keep, softmax, group_max, weight_scale)
   if (experts <= 64) MI355_ROUTE(1);
   else if (experts <= 128) MI355_ROUTE(2);
   else if (experts <= 256) MI355_ROUTE(4);
   else if (experts <= 512) MI355_ROUTE(8);
   else                                                  // one thread per token
     hipLaunchKernelGGL(moe_route_kernel, dim3(static_cast<unsigned>((num_tokens + 63) / 64)), dim3(64), 0, s, ids, weights,
-                       logits, correction, num_tokens, experts, top, groups, keep);
+                       logits, logits_stride, correction, num_tokens, experts, top, groups, keep, softmax, group_max,
+                       weight_scale);
 #undef MI355_ROUTE
   return check_launch("moe_route");
 }
@@ -461,7 +516,7 @@ extern "C" int32_t mi355_moe_gather_rows(void* xs, const void* x, const int32_t*
 
 extern "C" int32_t mi355_moe_gate_up_rows(void* act, const void* x, const void* w_gate_up, const int32_t* offsets,
                                           const int32_t* perm, int32_t experts, int32_t top, int32_t width, int32_t ff,
-                                          int32_t dtype, void* stream) {
+                                          int32_t act_fn, float limit, int32_t dtype, void* stream) {
   MI355_REQUIRE(act && x && w_gate_up && offsets && perm, MI355_ERR_INVALID, "moe_gate_up_rows: null pointer");
   MI355_REQUIRE(experts > 0 && experts <= 65535 && top > 0 && width > 0 && ff > 0, MI355_ERR_INVALID,
                 "moe_gate_up_rows: sizes");
@@ -472,10 +527,12 @@ extern "C" int32_t mi355_moe_gate_up_rows(void* act, const void* x, const void* 
     const dim3 mgrid(static_cast<unsigned>((ff / 16 + 3) / 4), static_cast<unsigned>(experts));
     if (dtype == MI355_BF16)
       hipLaunchKernelGGL((moe_gate_up_mfma_kernel<BF16>), mgrid, dim3(256), 0, s, static_cast<uint16_t*>(act),
-                         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w_gate_up), offsets, perm, top, width, ff);
+                         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w_gate_up), offsets, perm, top, width, ff,
+                         act_fn, limit);
     else
       hipLaunchKernelGGL((moe_gate_up_mfma_kernel<F16>), mgrid, dim3(256), 0, s, static_cast<uint16_t*>(act),
-                         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w_gate_up), offsets, perm, top, width, ff);
+                         static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(w_gate_up), offsets, perm, top, width, ff,
+                         act_fn, limit);
     return check_launch("moe_gate_up_rows (matrix cores)");
   }
   const bool vec = dtype != MI355_F32 && width % 8 == 0 && aligned16(x) && aligned16(w_gate_up);
@@ -483,11 +540,11 @@ extern "C" int32_t mi355_moe_gate_up_rows(void* act, const void* x, const void* 
     if (vec)
       hipLaunchKernelGGL((moe_gate_up_rows_kernel<TT, true>), grid, dim3(256), 0, s, static_cast<Elem<TT>::S*>(act),
                          static_cast<const Elem<TT>::S*>(x), static_cast<const Elem<TT>::S*>(w_gate_up), offsets, perm, top,
-                         width, ff);
+                         width, ff, act_fn, limit);
     else
       hipLaunchKernelGGL((moe_gate_up_rows_kernel<TT, false>), grid, dim3(256), 0, s, static_cast<Elem<TT>::S*>(act),
                          static_cast<const Elem<TT>::S*>(x), static_cast<const Elem<TT>::S*>(w_gate_up), offsets, perm, top,
-                         width, ff);
+                         width, ff, act_fn, limit);
   });
   return check_launch("moe_gate_up_rows");
 }
@@ -521,8 +578,8 @@ extern "C" int32_t mi355_moe_down_rows(void* y, const void* act, const void* w_d
   return check_launch("moe_down_rows");
 }
 
-extern "C" int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_rows, int32_t ff, int32_t dtype,
-                                          void* stream) {
+extern "C" int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_rows, int32_t ff, int32_t act, float limit,
+                                          int32_t dtype, void* stream) {
   MI355_REQUIRE(out && x, MI355_ERR_INVALID, "moe_silu_and_mul: null pointer");
   MI355_REQUIRE(num_rows >= 0 && ff > 0, MI355_ERR_INVALID, "moe_silu_and_mul: sizes");
   REQ_DTYPE(dtype);
@@ -532,14 +589,17 @@ extern "C" int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_
   const dim3 grid(static_cast<unsigned>(blocks > 65536 ? 65536 : blocks));
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_silu_and_mul_kernel<TT>), grid, dim3(256), 0, s,
                                                   static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(x),
-                                                  num_rows, ff));
+                                                  num_rows, ff, act, limit));
   return check_launch("moe_silu_and_mul");
 }
 
 extern "C" int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const float* weights, const int32_t* ids,
                                      const int32_t* offsets, int32_t pad_to, int64_t num_tokens, int32_t top, int32_t width,
-                                     int32_t dtype, void* stream) {
+                                     const void* x, int32_t num_real, const void* shared, const float* shared_gate,
+                                     int64_t shared_gate_stride, int32_t dtype, void* stream) {
   MI355_REQUIRE(out && y && inv && weights, MI355_ERR_INVALID, "moe_combine: null pointer");
+  MI355_REQUIRE(x == nullptr || (ids != nullptr && num_real >= 0), MI355_ERR_INVALID,
+                "moe_combine: identity experts need the chosen ids");
   MI355_REQUIRE(num_tokens >= 0 && top > 0 && width > 0 && pad_to >= 0 && (pad_to == 0 || (ids && offsets)), MI355_ERR_INVALID,
                 "moe_combine: sizes");
   REQ_DTYPE(dtype);
@@ -547,6 +607,8 @@ extern "C" int32_t mi355_moe_combine(void* out, const void* y, const int32_t* in
   hipStream_t s = static_cast<hipStream_t>(stream);
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((moe_combine_kernel<TT>), dim3(num_tokens), dim3(256), 0, s,
                                                   static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(y), inv,
-                                                  weights, ids, offsets, pad_to, top, width));
+                                                  weights, ids, offsets, pad_to, top, width,
+                                                  static_cast<const Elem<TT>::S*>(x), num_real,
+                                                  static_cast<const Elem<TT>::S*>(shared), shared_gate, shared_gate_stride));
   return check_launch("moe_combine");
 }

@@ -258,6 +258,85 @@ __global__ __launch_bounds__(256) void tanh_rows_kernel(typename Elem<T>::S* __r
     MI355_STF(T, out, out + i, tanhf(MI355_LDF(T, x, x + (i / n) * x_stride + i % n)));
 }
 
+// out[t] = embed[id] + bigram[row] + sinusoid(position), float32 rows.  row = (previous token * mul_prev
+// + id * mul_cur) mod buckets, `buckets` itself for a sequence's first token; the previous token of a
+// chunk's first row is the sequence's state (prev_tokens[slot], written by prev_token_update after
+// this launch).  Entry 2i of the sinusoid is sin(p * freq[i]), entry 2i + 1 the cosine; angles in fp32.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_bigram_pos_f32_kernel(
+    float* __restrict__ out, const typename Elem<T>::S* __restrict__ embed, const typename Elem<T>::S* __restrict__ bigram,
+    const int64_t* __restrict__ ids, const int64_t* __restrict__ positions, const int32_t* __restrict__ cu_seqlens,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ state_slots, const int32_t* __restrict__ prev_tokens,
+    const float* __restrict__ freq, int W, int64_t vocab, int64_t buckets, int64_t mul_prev, int64_t mul_cur) {
+  const int64_t t = blockIdx.x;
+  int64_t id = MI355_LD(int64_t, ids, ids + t);
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const int64_t p = MI355_LD(int64_t, positions, positions + t);
+  const typename Elem<T>::S* brow = nullptr;
+  if (bigram != nullptr) {
+    int64_t row = buckets;
+    if (p > 0) {
+      const int seq = MI355_LD(int32_t, tok_seq, tok_seq + t);
+      int64_t prev = t == MI355_LD(int32_t, cu_seqlens, cu_seqlens + seq)
+                         ? MI355_LD(int32_t, prev_tokens, prev_tokens + MI355_LD(int32_t, state_slots, state_slots + seq))
+                         : MI355_LD(int64_t, ids, ids + t - 1);
+      prev = prev < 0 ? 0 : (prev >= vocab ? vocab - 1 : prev);
+      row = (prev * mul_prev + id * mul_cur) % buckets;
+    }
+    brow = bigram + row * W;
+  }
+  const float pf = static_cast<float>(p);
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float v = MI355_LDF(T, embed, embed + id * W + c);
+    if (brow != nullptr) v += MI355_LDF(T, bigram, brow + c);
+    if (freq != nullptr) {
+      const float a = pf * MI355_LD(float, freq, freq + (c >> 1));
+      v += (c & 1) ? cosf(a) : sinf(a);
+    }
+    MI355_ST(float, out, out + t * W + c, v);
+  }
+}
+
+// prev_tokens[slot of chunk s] = the chunk's last token
+__global__ __launch_bounds__(256) void prev_token_update_kernel(int32_t* __restrict__ prev_tokens,
+                                                                const int64_t* __restrict__ ids,
+                                                                const int32_t* __restrict__ cu_seqlens,
+                                                                const int32_t* __restrict__ state_slots, int S) {
+  const int s = blockIdx.x * blockDim.x + threadIdx.x;
+  if (s >= S) return;
+  const int end = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s + 1);
+  if (end <= MI355_LD(int32_t, cu_seqlens, cu_seqlens + s)) return;
+  MI355_ST(int32_t, prev_tokens, prev_tokens + MI355_LD(int32_t, state_slots, state_slots + s),
+           static_cast<int32_t>(MI355_LD(int64_t, ids, ids + end - 1)));
+}
+
+// out = relu(x)^2
+template <typename T>
+__global__ __launch_bounds__(256) void relu_squared_kernel(typename Elem<T>::S* __restrict__ out,
+                                                           const typename Elem<T>::S* __restrict__ x, int64_t n) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const float v = fmaxf(MI355_LDF(T, x, x + i), 0.f);
+    MI355_STF(T, out, out + i, v * v);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void relu_squared_vec_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ x,
+                                                               int64_t nvec) {
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < nvec;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    float f[8];
+    unpack8<T>(MI355_LD(uint4, x, x + 8 * i), f);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float v = fmaxf(f[j], 0.f);
+      f[j] = v * v;
+    }
+    MI355_ST(uint4, out, out + 8 * i, pack8<T>(f));
+  }
+}
+
 static inline dim3 stride_grid(int64_t total) {
   const int64_t blocks = (total + 255) / 256;
   return dim3(static_cast<unsigned>(blocks < 1 ? 1 : (blocks > 65536 ? 65536 : blocks)));
@@ -279,6 +358,57 @@ extern "C" int32_t mi355_embed_scale_f32(float* out, const void* embed, const in
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((embed_scale_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s, out,
                                                   static_cast<const Elem<TT>::S*>(embed), ids, width, scale));
   return check_launch("embed_scale_f32");
+}
+
+extern "C" int32_t mi355_embed_bigram_pos_f32(float* out, const void* embed, const void* bigram, const int64_t* ids,
+                                              const int64_t* positions, const int32_t* cu_seqlens, const int32_t* tok_seq,
+                                              const int32_t* state_slots, const int32_t* prev_tokens, const float* freq,
+                                              int64_t num_tokens, int32_t width, int64_t vocab, int64_t buckets,
+                                              int64_t mul_prev, int64_t mul_cur, int32_t dtype, void* stream) {
+  MI355_REQUIRE(out && embed && ids && positions, MI355_ERR_INVALID, "embed_bigram_pos_f32: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && width > 0 && vocab > 0, MI355_ERR_INVALID, "embed_bigram_pos_f32: sizes");
+  MI355_REQUIRE(bigram == nullptr || (cu_seqlens && tok_seq && state_slots && prev_tokens && buckets > 0 && mul_prev >= 0 &&
+                                      mul_cur >= 0 && vocab <= (1ll << 31) && mul_prev < (1ll << 31) && mul_cur < (1ll << 31)),
+                MI355_ERR_INVALID, "embed_bigram_pos_f32: a bigram table needs the chunk layout, the state and its constants");
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((embed_bigram_pos_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s, out,
+                                                  static_cast<const Elem<TT>::S*>(embed),
+                                                  static_cast<const Elem<TT>::S*>(bigram), ids, positions, cu_seqlens,
+                                                  tok_seq, state_slots, prev_tokens, freq, width, vocab, buckets, mul_prev,
+                                                  mul_cur));
+  return check_launch("embed_bigram_pos_f32");
+}
+
+extern "C" int32_t mi355_prev_token_update(int32_t* prev_tokens, const int64_t* ids, const int32_t* cu_seqlens,
+                                           const int32_t* state_slots, int32_t num_seqs, void* stream) {
+  MI355_REQUIRE(prev_tokens && ids && cu_seqlens && state_slots, MI355_ERR_INVALID, "prev_token_update: null pointer");
+  MI355_REQUIRE(num_seqs >= 0, MI355_ERR_INVALID, "prev_token_update: sizes");
+  if (num_seqs == 0) return MI355_OK;
+  hipLaunchKernelGGL(prev_token_update_kernel, dim3((num_seqs + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     prev_tokens, ids, cu_seqlens, state_slots, num_seqs);
+  return check_launch("prev_token_update");
+}
+
+extern "C" int32_t mi355_relu_squared(void* out, const void* x, int64_t numel, int32_t dtype, void* stream) {
+  MI355_REQUIRE(out && x, MI355_ERR_INVALID, "relu_squared: null pointer");
+  MI355_REQUIRE(numel >= 0, MI355_ERR_INVALID, "relu_squared: sizes");
+  REQ_DTYPE(dtype);
+  if (numel == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype != MI355_F32 && numel % 8 == 0 && aligned16(out) && aligned16(x)) {
+    if (dtype == MI355_BF16)
+      hipLaunchKernelGGL((relu_squared_vec_kernel<BF16>), stride_grid(numel / 8), dim3(256), 0, s,
+                         static_cast<uint16_t*>(out), static_cast<const uint16_t*>(x), numel / 8);
+    else
+      hipLaunchKernelGGL((relu_squared_vec_kernel<F16>), stride_grid(numel / 8), dim3(256), 0, s,
+                         static_cast<uint16_t*>(out), static_cast<const uint16_t*>(x), numel / 8);
+    return check_launch("relu_squared");
+  }
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((relu_squared_kernel<TT>), stride_grid(numel), dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(x), numel));
+  return check_launch("relu_squared");
 }
 
 extern "C" int32_t mi355_resid_add_f32(float* resid, const float* other, const void* rows, const void* vec, int64_t num_tokens,

@@ -16,6 +16,8 @@
 //   conv_state_update       state <- the last taps-1 inputs of each sequence
 //   gated_delta_rule        S <- a S; u = b (v - S^T k); S <- S + k u^T; o = S^T q   per token and head
 //   general_delta_rule      S <- diag(w) S - (a * u) (u^T S) + k v^T; o = S^T r      per token and head
+//   mingru_scan             S <- (1 - z) S + z c per channel, z = sigmoid(zp + bz), c = u + 1/2 (u >= 0) or sigmoid(u),
+//                           u = xp + bx; out = S * silu(gp)
 #include "common.h"
 
 namespace mi355 {
@@ -821,6 +823,63 @@ __global__ __launch_bounds__(64) void general_delta_rule_cols_kernel(
   }
 }
 
+// A gated recurrence per channel whose gates read only the current token (zp, xp, gp: three column
+// ranges of the projection rows).  One workgroup per (64 channels, chunk); its waves take consecutive
+// segments of the chunk's rows.  The recurrence is linear in S, so a segment is summarised by
+// (A, B) with S_end = A S_start + B: every wave scans its segment from zero for (A, B), the
+// summaries of the earlier segments give its true start, and a second scan writes the outputs.  A
+// single wave (decoded tokens) scans once.  State, gates and candidates are fp32.
+template <typename T>
+__global__ __launch_bounds__(1024) void mingru_scan_kernel(
+    typename Elem<T>::S* __restrict__ out, const typename Elem<T>::S* __restrict__ proj, int64_t stride, int z_off, int x_off,
+    int g_off, const float* __restrict__ bz, const float* __restrict__ bx, float* __restrict__ state,
+    const int32_t* __restrict__ cu_seqlens, const int64_t* __restrict__ positions, const int32_t* __restrict__ state_slots,
+    int C) {
+  __shared__ float sa[16][64], sb[16][64];
+  const int s = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
+  const bool live = c < C;
+  const int r0 = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s), r1 = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s + 1);
+  if (r1 <= r0) return;                                 // (the whole workgroup)
+  const int per = (r1 - r0 + nw - 1) / nw;
+  const int a = r0 + wave * per < r1 ? r0 + wave * per : r1;
+  const int b = a + per < r1 ? a + per : r1;
+  const float zb = (live && bz != nullptr) ? MI355_LD(float, bz, bz + c) : 0.f;
+  const float xb = (live && bx != nullptr) ? MI355_LD(float, bx, bx + c) : 0.f;
+  auto gates = [&](int t, float& z, float& cand) {
+    const typename Elem<T>::S* row = proj + static_cast<int64_t>(t) * stride;
+    z = 1.0f / (1.0f + expf(-(MI355_LDF(T, proj, row + z_off + c) + zb)));
+    const float u = MI355_LDF(T, proj, row + x_off + c) + xb;
+    cand = u >= 0.f ? u + 0.5f : 1.0f / (1.0f + expf(-u));
+  };
+  if (nw > 1) {
+    float A = 1.0f, B = 0.f;
+    if (live) {
+      for (int t = a; t < b; ++t) {
+        float z, cand;
+        gates(t, z, cand);
+        A *= 1.0f - z;
+        B = (1.0f - z) * B + z * cand;
+      }
+    }
+    sa[wave][lane] = A;
+    sb[wave][lane] = B;
+    __syncthreads();
+  }
+  if (!live || a >= b) return;
+  const int64_t slot = MI355_LD(int32_t, state_slots, state_slots + s);
+  float S = MI355_LD(int64_t, positions, positions + r0) > 0 ? MI355_LD(float, state, state + slot * C + c) : 0.f;
+  for (int i = 0; i < wave; ++i) S = sa[i][lane] * S + sb[i][lane];
+  for (int t = a; t < b; ++t) {
+    float z, cand;
+    gates(t, z, cand);
+    S = (1.0f - z) * S + z * cand;
+    const float g = MI355_LDF(T, proj, proj + static_cast<int64_t>(t) * stride + g_off + c);
+    MI355_STF(T, out, out + static_cast<int64_t>(t) * C + c, S * (g / (1.0f + expf(-g))));
+  }
+  if (b == r1) MI355_ST(float, state, state + slot * C + c, S);
+}
+
 // out = sigmoid(gate) * sum of the key-range partial sums of sigmoid_window_attn_mfma_kernel
 template <typename T>
 __global__ __launch_bounds__(256) void window_attn_reduce_kernel(uint16_t* __restrict__ out, const float* __restrict__ partial,
@@ -1160,4 +1219,26 @@ extern "C" int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_s
   });
 #undef MI355_GDELTA
   return check_launch("general_delta_rule");
+}
+
+extern "C" int32_t mi355_mingru_scan(void* out, const void* proj, int64_t stride, int32_t z_off, int32_t x_off, int32_t g_off,
+                                     const float* z_bias, const float* x_bias, float* state, const int32_t* cu_seqlens,
+                                     const int64_t* positions, const int32_t* state_slots, int32_t num_seqs,
+                                     int64_t num_tokens, int32_t channels, int32_t long_chunks, int32_t dtype, void* stream) {
+  MI355_REQUIRE(out && proj && state && cu_seqlens && positions && state_slots, MI355_ERR_INVALID, "mingru_scan: null pointer");
+  MI355_REQUIRE(num_seqs >= 0 && num_seqs <= 65535 && num_tokens >= 0 && channels > 0 && z_off >= 0 && x_off >= 0 && g_off >= 0,
+                MI355_ERR_INVALID, "mingru_scan: sizes");
+  MI355_REQUIRE(stride >= static_cast<int64_t>(z_off) + channels && stride >= static_cast<int64_t>(x_off) + channels &&
+                    stride >= static_cast<int64_t>(g_off) + channels,
+                MI355_ERR_INVALID, "mingru_scan: rows shorter than the column ranges");
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0 || num_seqs == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>((channels + 63) / 64), static_cast<unsigned>(num_seqs));
+  const dim3 block(long_chunks ? 1024 : 64);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((mingru_scan_kernel<TT>), grid, block, 0, s,
+                                                  static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(proj), stride,
+                                                  z_off, x_off, g_off, z_bias, x_bias, state, cu_seqlens, positions,
+                                                  state_slots, channels));
+  return check_launch("mingru_scan");
 }

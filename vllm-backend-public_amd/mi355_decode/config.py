@@ -14,7 +14,7 @@ import os
 from dataclasses import dataclass, field
 from typing import Any, Optional
 
-SUPPORTED_ARCHS = ("LlamaForCausalLM", "Qwen2ForCausalLM", "MistralForCausalLM", "OPTForCausalLM", "Lozupel", "Tativik")
+SUPPORTED_ARCHS = ("LlamaForCausalLM", "Qwen2ForCausalLM", "MistralForCausalLM", "OPTForCausalLM", "Lozupel", "Tativik", "Tafisun")
 
 # Well-known geometries, used when --model names one of them and no local
 # config.json exists (synthetic-weight benchmarking; there is no network).
@@ -117,6 +117,62 @@ class MoESpec:
     groups: int
     keep: int
     ff: int
+    # what follows defaults to the first design that used this spec
+    score: str = "sigmoid"                  # "sigmoid": each expert by itself; "softmax": over all router outputs
+    group_score: str = "top2"               # a group scores the sum of its two best choice scores, or ("max") its best
+    weight_scale: float = 1.0               # the chosen experts' scores are multiplied by this
+    identity: int = 0                       # router outputs past `experts` that stand for "the input itself"; groups
+                                            # are formed over experts and identity outputs together
+    limit: Optional[float] = None           # None: silu(g) * u.  A number: g = min(g, limit), u = clamp(u, -limit, limit),
+                                            # g * sigmoid(1.702 g) * (u + 1)
+    shared_ff: int = 0                      # width of an expert that every token uses, scaled by a sigmoid of one
+    shared_limit: Optional[float] = None    # projected number per token; 0: none
+
+    @property
+    def outputs(self) -> int:
+        """Router outputs: experts and identity experts."""
+        return self.experts + self.identity
+
+    def check(self, where: str) -> None:
+        n = self.outputs
+        if self.experts < 1 or self.identity < 0 or n % self.groups or not 1 <= self.keep <= self.groups \
+                or not 1 <= self.top <= self.keep * (n // self.groups):
+            raise ValueError(f"{where}: {self.experts} experts + {self.identity} identity in {self.groups} groups, "
+                             f"{self.keep} kept, {self.top} chosen do not fit")
+
+
+@dataclass
+class BlockAttnSpec:
+    """Softmax attention inside blocks of `block` positions (position i sees j <= i with
+    i // block == j // block; block 0: plain causal), grouped heads, no rotation: the score is
+    q.k * scale - r1[h] * ln(1 + r2[h] * (i - j)).  Queries and keys get an RMS norm per head with one
+    weight vector shared by the heads.  values_are_keys: there is no value projection, the values
+    are the keys as projected, before their norm (then vdim == dim).  The concatenated heads are
+    multiplied by a sigmoid gate of their own width."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    block: int
+    scale: float
+    values_are_keys: bool = True
+
+
+@dataclass
+class MinGRUSpec:
+    """Gated recurrence over `width` channels whose gates read only the current token:
+    S <- (1 - z) S + z c, z = sigmoid(.), c = u + 1/2 for u >= 0 and sigmoid(u) below; the output is
+    S * silu(gate), projected."""
+    width: int
+
+
+@dataclass
+class BigramSpec:
+    """A second embedding table indexed by a hash of the previous and the current token:
+    row (prev * mul_prev + cur * mul_cur) mod buckets; the first token of a sequence takes row `buckets`."""
+    buckets: int
+    mul_prev: int
+    mul_cur: int
 
 
 @dataclass
@@ -130,6 +186,9 @@ class HybridLayerSpec:
     gdelta: Optional[GeneralDeltaSpec] = None
     lattn: Optional[LatentAttnSpec] = None
     moe: Optional[MoESpec] = None           # a mixture-of-experts feed-forward instead of a dense one
+    battn: Optional[BlockAttnSpec] = None   # kind "attention"
+    gru: Optional[MinGRUSpec] = None        # kind "mingru"
+    ff_act: str = "gelu_gated"              # the dense feed-forward: gelu_tanh(gate) * up, or "relu2": relu(up)^2, no gate
 
 
 @dataclass
@@ -150,6 +209,9 @@ class HybridSpec:
     arrangement: str = "pre"
     norm_groups: int = 1
     residual_mult: float = 1.0
+    norm_vector: bool = False               # "pre" arrangement: norms carry a weight per channel instead of one number
+    bigram: Optional[BigramSpec] = None     # a hashed previous-token embedding is added (the previous token is state)
+    sinusoid_base: float = 0.0              # > 0: sin / cos of pos * base^(-2i / width) in entries 2i / 2i + 1 is added
 
     def runs(self):
         """[(layer index, pass number or None)] in execution order: one cache / state each."""
@@ -160,6 +222,43 @@ class HybridSpec:
         for t in range(self.loop_times):
             out += [(i, t) for i in range(self.loop_start, self.loop_stop)]
         return out + [(i, None) for i in range(self.loop_stop, n)]
+
+    @classmethod
+    def from_tafisun(cls, d: dict) -> "HybridSpec":
+        layers = []
+        for i, spec in enumerate(d["layers"]):
+            m, mlp = spec["mixer"], spec.get("mlp")
+            kw = {}
+            if mlp is not None and mlp.get("kind", "dense") == "dense":
+                kw.update(ff=int(mlp["ff"]), ff_act="relu2")
+            elif mlp is not None and mlp.get("kind") == "moe":
+                r, sh = mlp["router"], mlp.get("shared") or None
+                g = r.get("groups") or {"count": 1, "keep": 1}
+                moe = MoESpec(experts=int(r["experts"]), top=int(r["top"]), groups=int(g.get("count", 1)),
+                              keep=int(g.get("keep", g.get("count", 1))), ff=int(mlp["expert"]["ff"]), score="softmax",
+                              group_score="max", weight_scale=float(r.get("scale", 1.0)), identity=int(r.get("identity", 0)),
+                              limit=float(mlp["expert"]["limit"]), shared_ff=int(sh["ff"]) if sh else 0,
+                              shared_limit=float(sh["limit"]) if sh else None)
+                moe.check(f"layer {i}")
+                kw.update(moe=moe)
+            elif mlp is not None:
+                raise ValueError(f"feed-forward kind {mlp.get('kind')!r} is not supported (dense, moe)")
+            if spec["type"] == "attention":
+                a = BlockAttnSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                                  vdim=int(m.get("vdim", m["dim"])), block=int((m.get("mask") or {}).get("size") or 0),
+                                  scale=float(m["scale"]))
+                if a.heads < 1 or a.kv_heads < 1 or a.heads % a.kv_heads:
+                    raise ValueError(f"layer {i}: kv_heads {a.kv_heads} must divide heads {a.heads}")
+                if a.vdim != a.dim:
+                    raise ValueError(f"layer {i}: the values are the keys, so vdim {a.vdim} must equal dim {a.dim}")
+                layers.append(HybridLayerSpec("attention", battn=a, **kw))
+            elif spec["type"] == "mingru":
+                layers.append(HybridLayerSpec("mingru", gru=MinGRUSpec(int(m["width"])), **kw))
+            else:
+                raise ValueError(f"layer type {spec['type']!r} is not supported (attention, mingru)")
+        b = (d.get("embedding") or {}).get("bigram")
+        return cls(layers=layers, norm_vector=True, sinusoid_base=10000.0,
+                   bigram=BigramSpec(int(b["buckets"]), int(b["mul_prev"]), int(b["mul_cur"])) if b else None)
 
     @classmethod
     def from_tativik(cls, d: dict) -> "HybridSpec":
@@ -281,6 +380,19 @@ class ModelConfig:
                    eos_token_id=d.get("eos_token_id"), family="hybrid", hybrid=spec)
 
     @classmethod
+    def _from_tafisun_dict(cls, d: dict) -> "ModelConfig":
+        spec = HybridSpec.from_tafisun(d)
+        att = [L.battn for L in spec.layers if L.battn is not None]
+        ffs = [L.ff or 0 for L in spec.layers] + [max(L.moe.ff, L.moe.shared_ff) for L in spec.layers if L.moe] + [0]
+        return cls(architecture="Tafisun", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]),
+                   intermediate_size=max(ffs), num_hidden_layers=len(spec.layers),
+                   num_attention_heads=max([a.heads for a in att] + [1]), num_key_value_heads=max([a.kv_heads for a in att] + [1]),
+                   head_dim=max([a.dim for a in att] + [1]), rope_theta=0.0, rope_scaling=None,
+                   rms_norm_eps=float(d["norm"]["eps"]), max_position_embeddings=int(d.get("max_positions", 1 << 17)),
+                   tie_word_embeddings=False, attention_bias=False, bos_token_id=d.get("bos_token_id"),
+                   eos_token_id=d.get("eos_token_id"), family="hybrid", hybrid=spec)
+
+    @classmethod
     def _from_tativik_dict(cls, d: dict) -> "ModelConfig":
         spec = HybridSpec.from_tativik(d)
         if int(d["width"]) % spec.norm_groups:
@@ -329,8 +441,9 @@ class ModelConfig:
             cfg = cls._from_opt_dict(d)
             cfg.torch_dtype = stored
             return cfg
-        if arch in ("Lozupel", "Tativik"):
-            cfg = cls._from_lozupel_dict(d) if arch == "Lozupel" else cls._from_tativik_dict(d)
+        if arch in ("Lozupel", "Tativik", "Tafisun"):
+            cfg = {"Lozupel": cls._from_lozupel_dict, "Tativik": cls._from_tativik_dict,
+                   "Tafisun": cls._from_tafisun_dict}[arch](d)
             cfg.torch_dtype = stored or "bfloat16"
             return cfg
         nh = d["num_attention_heads"]

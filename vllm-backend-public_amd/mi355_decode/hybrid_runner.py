@@ -3,6 +3,11 @@ mixer and may carry a feed-forward.  Two arrangements share this runner:
   * "pre" (the Lozupel design): a gated delta rule (a linear recurrence with a matrix state per
     head), or a sliding-window attention with sigmoid weights beside such a recurrence, and a dense
     gated feed-forward; a span of layers can run several times with shared weights;
+    a third design of this arrangement (Tafisun) adds a hashed previous-token embedding and
+    sinusoidal positions to the embedding, and mixes by a softmax attention inside blocks of positions
+    (logarithmic distance penalty, keys as values, normed queries and keys, a gate per output channel)
+    or by a per-channel gated recurrence; its feed-forward is relu^2 or a softmax-routed mixture with
+    identity experts and a shared expert;
   * "sandwich" (the Tativik design): a general delta rule (decay per key channel, removal along the
     unit key) or a softmax attention through low-rank latents (sliding window, a sink in the
     denominator, latent pages that a later layer may share), then a mixture of experts; every
@@ -159,8 +164,52 @@ class LatentAttention:
         return r.linear(o.transpose(0, 1).reshape(T, s.heads * s.vdim), lw.o_w)
 
 
+class BlockAttention:
+    """Softmax attention inside blocks of positions with a logarithmic distance penalty over the paged
+    K/V of one layer run.  Queries and keys are RMS-normed per head; the V pages hold the keys as
+    projected (the design has no value projection)."""
+
+    def __init__(self, spec, lw, runner, cache_index: int):
+        self.s, self.lw, self.r, self.ci = spec, lw, runner, cache_index
+
+    def __call__(self, proj: torch.Tensor, b: StepBatch) -> torch.Tensor:
+        s, lw, r = self.s, self.lw, self.r
+        col = lambda n: proj[:, lw.seg[n][0]: lw.seg[n][0] + lw.seg[n][1]]     # noqa: E731
+        q, k = col("q"), col("k")
+        kc, vc = r.k_cache[self.ci], r.v_cache[self.ci]
+        ops.qk_norm_kv_write(q, k, k, lw.q_norm, lw.k_norm, b.slot_mapping, kc, vc, s.heads, s.kv_heads, s.dim, s.vdim, r.eps)
+        o = ops.softmax_bias_attn(q, kc, vc, b.block_tables, b.tok_seq, b.positions, lw.r1, lw.r2, col("g"), s.heads,
+                                  s.scale, block=s.block, tiles=b.tiles, num_splits=r.block_key_splits(b, s))
+        return r.linear(o, lw.o_w)
+
+
+class MinGRUMixer:
+    """Per-channel gated recurrence on one layer run's state slots: gates and candidate from the
+    current token only, the state in float32."""
+
+    def __init__(self, spec, lw, runner, state_index: int):
+        self.s, self.lw, self.r, self.si = spec, lw, runner, state_index
+
+    def __call__(self, proj: torch.Tensor, b: StepBatch) -> torch.Tensor:
+        lw, seg = self.lw, self.lw.seg
+        o = ops.mingru_scan(proj, seg["z"][0], seg["x"][0], seg["g"][0], self.s.width, lw.z_b, lw.x_b,
+                            self.r.rec_state[self.si], b.cu_seqlens, b.positions, b.state_slots, long_chunks=b.long_chunks)
+        return self.r.linear(o, lw.o_w)
+
+
+class ReluSquaredFF:
+    """Dense feed-forward without a gate: down(relu(up h)^2)."""
+
+    def __init__(self, lw, runner):
+        self.lw, self.r = lw, runner
+
+    def __call__(self, h: torch.Tensor) -> torch.Tensor:
+        return self.r.linear(ops.relu_squared(self.r.linear(h, self.lw.up_w)), self.lw.down_w)
+
+
 class MoEFeedForward:
-    """Mixture of experts: fp32 routing, rows sorted by expert, the expert products, the weighted sum."""
+    """Mixture of experts: fp32 routing, rows sorted by expert, the expert products, the weighted sum
+    (which also takes in identity experts and a gated shared expert where the design has them)."""
 
     GROUPED_MIN_ROWS = 512          # from this many routed rows on, one library GEMM per expert (needs the counts on the host)
 
@@ -181,39 +230,53 @@ class MoEFeedForward:
             out[a: a + self.GROUPED_MAX_TOKENS] = self._tokens(h[a: a + self.GROUPED_MAX_TOKENS])
         return out
 
+    def _act(self, gu: torch.Tensor, limit, ff: int) -> torch.Tensor:
+        if limit is None and gu.dtype != torch.float32 and ff % 8 == 0:
+            return ops.silu_and_mul(gu)
+        return ops.moe_silu_and_mul(gu, limit)
+
     def _tokens(self, h: torch.Tensor) -> torch.Tensor:
         s, lw = self.s, self.lw
-        T = h.shape[0]
-        ids, wts = ops.moe_route(torch.mm(h.float(), lw.router_w.t()), lw.correction, s.top, s.groups, s.keep)
-        offsets, perm, inv = ops.moe_sort(ids, s.experts)
+        T, E = h.shape[0], s.experts
+        # the router product in fp32; a shared expert's gate is one more row of the same matrix
+        logits = torch.mm(h.float(), lw.router_w.t())
+        ids, wts = ops.moe_route(logits, lw.correction, s.top, s.groups, s.keep, softmax=s.score == "softmax",
+                                 group_max=s.group_score == "max", weight_scale=s.weight_scale, experts=s.outputs)
+        offsets, perm, inv = ops.moe_sort(ids, s.outputs)
+        extra = {}
+        if s.identity:
+            extra.update(ids=ids, x=h, num_real=E)
+        if s.shared_ff:
+            gu = self.r.linear(h, lw.shared_gate_up_w)
+            extra.update(shared=self.r.linear(self._act(gu, s.shared_limit, s.shared_ff), lw.shared_down_w),
+                         shared_gate=logits[:, s.outputs:])
         rows = T * s.top
         if rows >= self.GROUPED_MIN_ROWS and not torch.cuda.is_current_stream_capturing():
-            # many rows: library GEMMs per expert.  The largest count comes to the host (one wait); when the
-            # experts' loads are near even, every expert's rows are padded to that count and the two products
+            # many rows: library GEMMs per expert.  The experts' row ranges come to the host (one wait); when
+            # the loads are near even, every expert's rows are padded to the largest count and the two products
             # are one batched GEMM each; otherwise one GEMM per expert on its range of the sorted rows.
-            counts = offsets[1:] - offsets[:-1]
-            cap = -(-int(counts.max()) // 16) * 16
-            if s.experts * cap <= 2 * rows:
-                xp = ops.moe_gather_rows(h, perm, rows, s.top, offsets=offsets, pad_to=cap)
-                gu = torch.bmm(xp.view(s.experts, cap, -1), lw.gate_up_w.transpose(1, 2)).view(s.experts * cap, 2 * s.ff)
-                act = ops.silu_and_mul(gu) if h.dtype != torch.float32 and s.ff % 8 == 0 else ops.moe_silu_and_mul(gu)
-                y = torch.bmm(act.view(s.experts, cap, s.ff), lw.down_w.transpose(1, 2)).view(s.experts * cap, -1)
-                return ops.moe_combine(y, inv, wts, T, s.top, ids=ids, offsets=offsets, pad_to=cap)
-            else:
-                xs = ops.moe_gather_rows(h, perm, rows, s.top)
-                off = offsets.tolist()
-                gu = torch.empty(rows, 2 * s.ff, dtype=h.dtype, device=h.device)
-                for e in range(s.experts):
-                    if off[e + 1] > off[e]:
-                        torch.mm(xs[off[e]: off[e + 1]], lw.gate_up_w[e].t(), out=gu[off[e]: off[e + 1]])
-                act = ops.moe_silu_and_mul(gu)
-                y = torch.empty(rows, h.shape[1], dtype=h.dtype, device=h.device)
-                for e in range(s.experts):
-                    if off[e + 1] > off[e]:
-                        torch.mm(act[off[e]: off[e + 1]], lw.down_w[e].t(), out=y[off[e]: off[e + 1]])
+            off = offsets.tolist()
+            cap = -(-max(off[e + 1] - off[e] for e in range(E)) // 16) * 16
+            if 0 < E * cap <= 2 * off[E]:
+                xp = ops.moe_gather_rows(h, perm, rows, s.top, offsets=offsets, pad_to=cap, experts=E)
+                gu = torch.bmm(xp.view(E, cap, -1), lw.gate_up_w.transpose(1, 2)).view(E * cap, 2 * s.ff)
+                y = torch.bmm(self._act(gu, s.limit, s.ff).view(E, cap, s.ff), lw.down_w.transpose(1, 2)).view(E * cap, -1)
+                extra["ids"] = ids
+                return ops.moe_combine(y, inv, wts, T, s.top, offsets=offsets, pad_to=cap, **extra)
+            xs = ops.moe_gather_rows(h, perm, rows, s.top)
+            gu = torch.empty(rows, 2 * s.ff, dtype=h.dtype, device=h.device)
+            for e in range(E):
+                if off[e + 1] > off[e]:
+                    torch.mm(xs[off[e]: off[e + 1]], lw.gate_up_w[e].t(), out=gu[off[e]: off[e + 1]])
+            act = ops.moe_silu_and_mul(gu, s.limit)
+            y = torch.empty(rows, h.shape[1], dtype=h.dtype, device=h.device)
+            for e in range(E):
+                if off[e + 1] > off[e]:
+                    torch.mm(act[off[e]: off[e + 1]], lw.down_w[e].t(), out=y[off[e]: off[e + 1]])
         else:
-            y = ops.moe_down_rows(ops.moe_gate_up_rows(h, lw.gate_up_w, offsets, perm, s.top), lw.down_w, offsets)
-        return ops.moe_combine(y, inv, wts, T, s.top)
+            y = ops.moe_down_rows(ops.moe_gate_up_rows(h, lw.gate_up_w, offsets, perm, s.top, limit=s.limit), lw.down_w,
+                                  offsets)
+        return ops.moe_combine(y, inv, wts, T, s.top, **extra)
 
 
 class HybridRunner(ModelRunner):
@@ -278,6 +341,18 @@ class HybridRunner(ModelRunner):
             self.ffs.append(MoEFeedForward(L.moe, lw, self) if L.moe is not None else None)
         for li, _ in self.runs if spec.arrangement != "sandwich" else ():
             L, lw = spec.layers[li], weights.layers[li]
+            self.ffs.append(MoEFeedForward(L.moe, lw, self) if L.moe is not None else
+                            ReluSquaredFF(lw, self) if L.ff and L.ff_act == "relu2" else None)
+            if L.kind == "attention":
+                A = L.battn
+                self.k_cache.append(torch.zeros(self.num_blocks, A.kv_heads, BLOCK_SIZE, A.dim, dtype=dtype, device=dev))
+                self.v_cache.append(torch.zeros(self.num_blocks, A.kv_heads, A.vdim, BLOCK_SIZE, dtype=dtype, device=dev))
+                self.mixers.append(BlockAttention(A, lw, self, len(self.k_cache) - 1))
+                continue
+            if L.kind == "mingru":
+                self.rec_state.append(torch.zeros(self.num_state_slots + 1, L.gru.width, dtype=torch.float32, device=dev))
+                self.mixers.append(MinGRUMixer(L.gru, lw, self, len(self.rec_state) - 1))
+                continue
             D = L.delta
             attn = None
             if L.attn is not None:
@@ -291,6 +366,14 @@ class HybridRunner(ModelRunner):
             self.rec_state.append(torch.zeros(self.num_state_slots + 1, D.heads, D.dim, D.vdim, dtype=torch.float32,
                                               device=dev))
             self.mixers.append((attn, DeltaMixer(D, lw, self, len(self.rec_state) - 1)))
+        # the previous token of every live sequence (hashed previous-token embedding), beside the other state
+        self.prev_tokens = torch.zeros(self.num_state_slots + 1, dtype=torch.int32, device=dev) \
+            if spec.bigram is not None else None
+        self._pos_freq = None
+        if spec.sinusoid_base > 0:
+            half = (self.H + 1) // 2
+            f = float(spec.sinusoid_base) ** (-2.0 * np.arange(half, dtype=np.float64) / self.H)
+            self._pos_freq = torch.from_numpy(f.astype(np.float32)).to(dev)
         B = self.max_num_seqs
         self._init_step_inputs(extra_i32=1)
         self.row_extra.fill_(self.num_state_slots)
@@ -355,12 +438,24 @@ class HybridRunner(ModelRunner):
             return {"partial": self._attn_partial, "num_splits": n}      # static: a decode graph holds its address
         return {"partial": torch.empty(need, dtype=torch.float32, device=self.device), "num_splits": n}
 
+    def block_key_splits(self, b: StepBatch, a) -> int:
+        """Workgroups per tile for the block attention (as key_splits: decoded tokens and short prompts)."""
+        if b.tiles is None or self.dtype == torch.float32:
+            return 0
+        rep = a.heads // a.kv_heads
+        hb = 4 if rep % 4 == 0 else 3 if rep % 3 == 0 else 2 if rep % 2 == 0 else 1
+        waves = int(b.tiles.shape[0]) * a.kv_heads * (rep // hb)
+        span = a.block if a.block > 0 else self.max_model_len
+        n = min(self.MAX_KEY_SPLITS, max(span // 64, 1), max(2048 // max(waves, 1), 1))
+        return n if n > 1 else 0
+
     def kv_cache_bytes_per_block(self) -> int:
         pages = self.k_cache + self.v_cache + [t for pair in self.latent_cache for t in pair if t is not None]
         return sum(t[0].numel() * t.element_size() for t in pages)
 
     def state_bytes_per_slot(self) -> int:
-        return sum(t[0].numel() * t.element_size() for t in self.conv_state + self.rec_state)
+        return sum(t[0].numel() * t.element_size() for t in self.conv_state + self.rec_state) \
+            + (4 if self.prev_tokens is not None else 0)
 
     def _init_tiled_copies(self, want: Optional[bool]) -> None:
         """Fragment-tiled second copies of the wide matrices for the weight-streaming GEMM of decode-sized
@@ -373,7 +468,7 @@ class HybridRunner(ModelRunner):
         mats = [self.head_w]
         for lw in self.w.layers:
             mats += [getattr(lw, n, None) for n in ("in_w", "delta_o_w", "attn_o_w", "gate_up_w", "down_w", "a2_w", "g2_w",
-                                                    "o_w", "uq_w", "w2_w", "rg2_w")]
+                                                    "o_w", "uq_w", "w2_w", "rg2_w", "up_w", "shared_gate_up_w", "shared_down_w")]
         for w in mats:
             # the kernel stages x in 512-wide K slices; narrow outputs leave too few workgroups to pay
             if w is not None and w.dim() == 2 and w.shape[1] % 512 == 0 and w.shape[0] >= 256 and w.shape[0] % 8 == 0:
@@ -450,7 +545,15 @@ class HybridRunner(ModelRunner):
     def _forward_pre(self, b: StepBatch) -> torch.Tensor:
         """All layers over one packed batch; returns the float32 residual stream [tokens, width]."""
         w, spec = self.w, self.spec
-        resid = ops.embed_scale_f32(w.embed, b.ids, spec.embed_scale)
+        if spec.bigram is not None or self._pos_freq is not None:
+            bg = spec.bigram
+            resid = ops.embed_bigram_pos_f32(w.embed, b.ids, b.positions, w.bigram,
+                                             (bg.buckets, bg.mul_prev, bg.mul_cur) if bg else None, b.cu_seqlens, b.tok_seq,
+                                             b.state_slots, self.prev_tokens, self._pos_freq)
+            if bg is not None:
+                ops.prev_token_update(self.prev_tokens, b.ids, b.cu_seqlens, b.state_slots)
+        else:
+            resid = ops.embed_scale_f32(w.embed, b.ids, spec.embed_scale)
         x0 = resid.clone() if spec.loop_times > 1 else None
         pending = None                                 # a sub-layer output not yet added to the residual
         last = len(self.runs) - 1
@@ -462,13 +565,18 @@ class HybridRunner(ModelRunner):
             h = ops.add_rms_norm_f32(resid, lw.norm1, self.eps, add=pending)    # the add rides in the norm's launch
             pending = None
             proj = self.linear(h, lw.in_w)
-            attn, delta = self.mixers[ri]
-            if attn is not None:
+            mixer, ff = self.mixers[ri], self.ffs[ri]
+            if not isinstance(mixer, tuple):
+                pending = mixer(proj, b)
+            elif mixer[0] is not None:
+                attn, delta = mixer
                 ops.rms_norm_mix_f32(resid, attn(proj, b), lw.attn_out_norm, delta(proj, b), lw.delta_out_norm,
                                      self.eps, 0.5)
             else:
-                pending = delta(proj, b)
-            if L.ff:
+                pending = mixer[1](proj, b)
+            if ff is not None:
+                pending = ff(ops.add_rms_norm_f32(resid, lw.norm2, self.eps, add=pending))
+            elif L.ff:
                 h = ops.add_rms_norm_f32(resid, lw.norm2, self.eps, add=pending)
                 pending = self.linear(ops.gelu_tanh_and_mul(self.linear(h, lw.gate_up_w)), lw.down_w)
             if pending is not None and (ri == last or self.layer_trace is not None):

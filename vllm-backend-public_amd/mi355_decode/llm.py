@@ -62,7 +62,7 @@ def plan_num_blocks(args: EngineArgs, cfg: ModelConfig, tp_size: int, num_layers
     per_block = 2 * num_layers * (cfg.num_key_value_heads // tp_size) * BLOCK_SIZE * cfg.head_dim * elem_size
     if cfg.family == "hybrid":                        # K and V pages of every layer run that has an attention
         runs = [cfg.hybrid.layers[i] for i, _ in cfg.hybrid.runs()]
-        per_tok = sum(L.attn.kv_heads * (L.attn.dim + L.attn.vdim) for L in runs if L.attn is not None)
+        per_tok = sum(a.kv_heads * (a.dim + a.vdim) for L in runs for a in (L.attn, L.battn) if a is not None)
         # a latent attention caches its latent and one rotated key part, unless it reads another layer's
         # (in 16 bits the latent twice: token-major for the scores, channel-major for the weighted sum)
         per_tok += sum((1 if elem_size == 4 else 2) * L.lattn.kv_rank + L.lattn.rot_dim for L in runs

@@ -1393,13 +1393,22 @@ def latent_window_attn(q_latent: torch.Tensor, q: torch.Tensor, q_head_width: in
     return out
 
 
-def moe_route(logits: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int):
-    """float32 router logits [tokens, experts] -> (ids int32 [tokens, top], weights float32 [tokens, top])."""
-    T, E = logits.shape
+def moe_route(logits: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int, softmax: bool = False,
+              group_max: bool = False, weight_scale: float = 1.0, experts: int | None = None):
+    """float32 router logits [tokens, >= experts] (rows may carry more columns than router outputs:
+    `experts` says how many count) -> (ids int32 [tokens, top], weights float32 [tokens, top]).
+    Scores are a sigmoid per logit or (softmax) a softmax over the router outputs; a group scores the
+    sum of its two best choice scores or (group_max) its best."""
+    T = logits.shape[0]
+    E = int(experts) if experts is not None else logits.shape[1]
+    _dev(logits, "logits")
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1 or logits.shape[1] < E:
+        raise ValueError("logits must be float32 [tokens, >= experts] with a contiguous last dim")
     ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
     wts = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-    check(lib.mi355_moe_route(ids.data_ptr(), wts.data_ptr(), _f32(logits, "logits"), _f32(correction, "correction", E),
-                              T, E, int(top), int(groups), int(keep), _stream()))
+    check(lib.mi355_moe_route(ids.data_ptr(), wts.data_ptr(), logits.data_ptr(), logits.stride(0) if T > 1 else logits.shape[1],
+                              _f32(correction, "correction", E), T, E, int(top), int(groups), int(keep), int(bool(softmax)),
+                              int(bool(group_max)), float(weight_scale), _stream()))
     return ids, wts
 
 
@@ -1416,13 +1425,13 @@ def moe_sort(ids: torch.Tensor, experts: int):
 
 
 def moe_gather_rows(x: torch.Tensor, perm: torch.Tensor, rows: int, top: int, offsets: torch.Tensor | None = None,
-                    pad_to: int = 0):
+                    pad_to: int = 0, experts: int | None = None):
     """The routed rows of x in expert order [rows, width]; with pad_to > 0 every expert's rows padded
-    with zero rows to pad_to: [experts * pad_to, width]."""
+    with zero rows to pad_to: [experts * pad_to, width] (`experts`: the first so many of offsets')."""
     dt = _dt3(x, "x")
     if not x.is_contiguous():
         raise ValueError("x must be contiguous")
-    n = rows if pad_to <= 0 else (offsets.numel() - 1) * pad_to
+    n = rows if pad_to <= 0 else (int(experts) if experts is not None else offsets.numel() - 1) * pad_to
     xs = torch.empty(n, x.shape[1], dtype=x.dtype, device=x.device)
     check(lib.mi355_moe_gather_rows(xs.data_ptr(), x.data_ptr(), _idx(perm, "perm", torch.int32, rows),
                                     None if pad_to <= 0 else _idx(offsets, "offsets", torch.int32), max(int(pad_to), 0), n,
@@ -1430,17 +1439,28 @@ def moe_gather_rows(x: torch.Tensor, perm: torch.Tensor, rows: int, top: int, of
     return xs
 
 
-def moe_gate_up_rows(x: torch.Tensor, w_gate_up: torch.Tensor, offsets: torch.Tensor, perm: torch.Tensor, top: int):
-    """silu(Wg[e] x) * (Wu[e] x) for every routed row, in expert order: [tokens * top, ff]."""
+ACT_SILU_MUL, ACT_LIMITED = 0, 1
+
+
+def _gate_act(limit) -> tuple:
+    return (ACT_SILU_MUL, 0.0) if limit is None else (ACT_LIMITED, float(limit))
+
+
+def moe_gate_up_rows(x: torch.Tensor, w_gate_up: torch.Tensor, offsets: torch.Tensor, perm: torch.Tensor, top: int,
+                     limit: float | None = None):
+    """a(Wg[e] x, Wu[e] x) for every routed row, in expert order: [tokens * top, ff].  a(g, u) is
+    silu(g) * u, or with a limit g' sigmoid(1.702 g') (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit).
+    offsets may list more bins than w_gate_up has experts (identity experts): their rows are left alone."""
     dt = _dt3(x, "x")
     E, F2, W = w_gate_up.shape
     if not x.is_contiguous() or x.shape[1] != W or not w_gate_up.is_contiguous():
         raise ValueError("x must be contiguous [tokens, width], w_gate_up contiguous [experts, 2 ff, width]")
     rows = x.shape[0] * top
     act = torch.empty(rows, F2 // 2, dtype=x.dtype, device=x.device)
+    fn, lim = _gate_act(limit)
     check(lib.mi355_moe_gate_up_rows(act.data_ptr(), x.data_ptr(), _same(w_gate_up, x, "w_gate_up"),
                                      _idx(offsets, "offsets", torch.int32, E + 1), _idx(perm, "perm", torch.int32, rows),
-                                     E, int(top), W, F2 // 2, dt, _stream()))
+                                     E, int(top), W, F2 // 2, fn, lim, dt, _stream()))
     return act
 
 
@@ -1455,27 +1475,173 @@ def moe_down_rows(act: torch.Tensor, w_down: torch.Tensor, offsets: torch.Tensor
     return y
 
 
-def moe_silu_and_mul(x: torch.Tensor):
+def moe_silu_and_mul(x: torch.Tensor, limit: float | None = None):
+    """x [rows, 2 ff] holding gate | up -> a(gate, up) (see moe_gate_up_rows)."""
     dt = _dt3(x, "x")
     if not x.is_contiguous():
         raise ValueError("x must be contiguous [rows, 2 ff]")
     out = torch.empty(x.shape[0], x.shape[1] // 2, dtype=x.dtype, device=x.device)
-    check(lib.mi355_moe_silu_and_mul(out.data_ptr(), x.data_ptr(), x.shape[0], x.shape[1] // 2, dt, _stream()))
+    fn, lim = _gate_act(limit)
+    check(lib.mi355_moe_silu_and_mul(out.data_ptr(), x.data_ptr(), x.shape[0], x.shape[1] // 2, fn, lim, dt, _stream()))
     return out
 
 
 def moe_combine(y: torch.Tensor, inv: torch.Tensor, weights: torch.Tensor, num_tokens: int, top: int,
-                ids: torch.Tensor | None = None, offsets: torch.Tensor | None = None, pad_to: int = 0):
+                ids: torch.Tensor | None = None, offsets: torch.Tensor | None = None, pad_to: int = 0,
+                x: torch.Tensor | None = None, num_real: int = 0, shared: torch.Tensor | None = None,
+                shared_gate: torch.Tensor | None = None):
     """out[t] = sum_k weights[t, k] * y[inv[t * top + k]]; with pad_to > 0, y holds every expert's rows
-    padded to pad_to (moe_gather_rows) and ids / offsets locate them."""
+    padded to pad_to (moe_gather_rows) and ids / offsets locate them.  x: chosen ids >= num_real are
+    identity experts whose row is x[t].  shared [tokens, width]: added, times the sigmoid of
+    shared_gate (float32, one number per token; any row stride) if given."""
     dt = _dt3(y, "y")
     if not y.is_contiguous():
         raise ValueError("y must be contiguous")
-    out = torch.empty(num_tokens, y.shape[1], dtype=y.dtype, device=y.device)
+    W = y.shape[1]
+    out = torch.empty(num_tokens, W, dtype=y.dtype, device=y.device)
     pad = max(int(pad_to), 0)
+    need_ids = pad > 0 or x is not None
+    for n, t in (("x", x), ("shared", shared)):
+        if t is not None and (t.dtype != y.dtype or not t.is_contiguous() or tuple(t.shape) != (num_tokens, W)):
+            raise ValueError(f"{n} must be contiguous [tokens, width] in the dtype of y")
+    sg, sgs = None, 0
+    if shared_gate is not None:
+        _dev(shared_gate, "shared_gate")
+        if shared is None or shared_gate.dtype != torch.float32 or shared_gate.shape[0] != num_tokens:
+            raise ValueError("shared_gate: float32, one number per token, with shared rows")
+        sg, sgs = shared_gate.data_ptr(), (shared_gate.stride(0) if num_tokens > 1 else 1)
     check(lib.mi355_moe_combine(out.data_ptr(), y.data_ptr(), _idx(inv, "inv", torch.int32, num_tokens * top),
                                 _f32(weights, "weights", num_tokens * top),
-                                None if pad == 0 else _idx(ids, "ids", torch.int32, num_tokens * top),
+                                None if not need_ids else _idx(ids, "ids", torch.int32, num_tokens * top),
                                 None if pad == 0 else _idx(offsets, "offsets", torch.int32), pad, num_tokens, int(top),
-                                y.shape[1], dt, _stream()))
+                                W, None if x is None else x.data_ptr(), int(num_real),
+                                None if shared is None else shared.data_ptr(), sg, sgs, dt, _stream()))
+    return out
+
+
+# ---- hashed previous-token embedding, block attention with a distance penalty, per-channel gated recurrence
+def embed_bigram_pos_f32(embed: torch.Tensor, ids: torch.Tensor, positions: torch.Tensor, bigram: torch.Tensor | None = None,
+                         hash_consts: tuple | None = None, cu_seqlens: torch.Tensor | None = None,
+                         tok_seq: torch.Tensor | None = None, state_slots: torch.Tensor | None = None,
+                         prev_tokens: torch.Tensor | None = None, freq: torch.Tensor | None = None):
+    """float32 rows embed[id] + bigram[(prev * mul_prev + id * mul_cur) % buckets] + sinusoid(position).
+    hash_consts = (buckets, mul_prev, mul_cur); bigram [buckets + 1, width], its last row for position
+    0.  The previous token of a chunk's first row is prev_tokens[state slot] (int32; see
+    prev_token_update).  freq float32 [ceil(width / 2)]: entries 2i / 2i + 1 get sin / cos of
+    position * freq[i]."""
+    dt = _dt3(embed, "embed")
+    if embed.dim() != 2 or not embed.is_contiguous():
+        raise ValueError("embed must be contiguous [vocab, width]")
+    T, W = ids.numel(), embed.shape[1]
+    out = torch.empty(T, W, dtype=torch.float32, device=embed.device)
+    buckets = mp = mc = 0
+    if bigram is not None:
+        buckets, mp, mc = (int(v) for v in hash_consts)
+        if bigram.dtype != embed.dtype or not bigram.is_contiguous() or tuple(bigram.shape) != (buckets + 1, W):
+            raise ValueError("bigram must be contiguous [buckets + 1, width] in the dtype of embed")
+        S = cu_seqlens.numel() - 1
+        _idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(tok_seq, "tok_seq", torch.int32, T)
+        _idx(state_slots, "state_slots", torch.int32, S), _idx(prev_tokens, "prev_tokens", torch.int32)
+    if freq is not None:
+        _f32(freq, "freq", (W + 1) // 2)
+    check(lib.mi355_embed_bigram_pos_f32(
+        out.data_ptr(), embed.data_ptr(), None if bigram is None else bigram.data_ptr(), _idx(ids, "ids", torch.int64),
+        _idx(positions, "positions", torch.int64, T), None if bigram is None else cu_seqlens.data_ptr(),
+        None if bigram is None else tok_seq.data_ptr(), None if bigram is None else state_slots.data_ptr(),
+        None if bigram is None else prev_tokens.data_ptr(), None if freq is None else freq.data_ptr(), T, W, embed.shape[0],
+        buckets, mp, mc, dt, _stream()))
+    return out
+
+
+def prev_token_update(prev_tokens: torch.Tensor, ids: torch.Tensor, cu_seqlens: torch.Tensor, state_slots: torch.Tensor):
+    """prev_tokens[state slot of chunk s] = the last token of chunk s."""
+    S = cu_seqlens.numel() - 1
+    check(lib.mi355_prev_token_update(_idx(prev_tokens, "prev_tokens", torch.int32), _idx(ids, "ids", torch.int64),
+                                      _idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(state_slots, "state_slots", torch.int32, S),
+                                      S, _stream()))
+    return prev_tokens
+
+
+def relu_squared(x: torch.Tensor):
+    """max(x, 0)^2."""
+    dt = _dt3(x, "x")
+    if not x.is_contiguous():
+        raise ValueError("x must be contiguous")
+    out = torch.empty_like(x)
+    check(lib.mi355_relu_squared(out.data_ptr(), x.data_ptr(), x.numel(), dt, _stream()))
+    return out
+
+
+def qk_norm_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor,
+                     slot_mapping: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, num_heads: int,
+                     num_kv_heads: int, head_dim: int, v_dim: int, eps: float):
+    """q [tokens, heads * dim] is RMS-normed per head in place (weight float32 [dim]); the normed k goes
+    to the K pages, v (as given; it may be k itself) to the V pages.  q / k / v may be column slices."""
+    dt = _dt3(q, "q")
+    T = q.shape[0]
+    check(lib.mi355_qk_norm_kv_write(
+        q.data_ptr(), _cols(q, "q", num_heads * head_dim), _same(k, q, "k"), _cols(k, "k", num_kv_heads * head_dim),
+        _same(v, q, "v"), _cols(v, "v", num_kv_heads * v_dim), _f32(q_weight, "q_weight", head_dim),
+        _f32(k_weight, "k_weight", head_dim), _idx(slot_mapping, "slot_mapping", torch.int64, T),
+        _same(k_cache, q, "k_cache"), _same(v_cache, q, "v_cache"), T, num_heads, num_kv_heads, head_dim, v_dim, float(eps),
+        dt, _stream()))
+
+
+def softmax_bias_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                      tok_seq: torch.Tensor, positions: torch.Tensor, r1: torch.Tensor | None, r2: torch.Tensor | None,
+                      gate: torch.Tensor | None, num_heads: int, scale: float, block: int = 0, window: int = 0,
+                      tiles: torch.Tensor | None = None, num_splits: int = 0):
+    """Softmax attention over the paged K/V [blocks, kv_heads, 16, dim] / [blocks, kv_heads, vdim, 16] with
+    the score q.k * scale - r1[h] ln(1 + r2[h] * distance); a row at position p sees the keys j <= p of
+    its block of `block` positions (0: all) and, window > 0, the last `window` of them.  gate
+    [tokens, heads] or [tokens, heads * vdim]: the output is multiplied by its sigmoid.  tiles
+    (query_tiles) selects the matrix-core form where the sizes allow; num_splits > 1 spreads a
+    tile's keys over that many workgroups.  Returns [tokens, heads * vdim]."""
+    dt = _dt3(q, "q")
+    T = q.shape[0]
+    G, d, dv = k_cache.shape[1], k_cache.shape[3], v_cache.shape[2]
+    if k_cache.shape[2] != BLOCK_SIZE or v_cache.shape[3] != BLOCK_SIZE or v_cache.shape[1] != G \
+            or not k_cache.is_contiguous() or not v_cache.is_contiguous():
+        raise ValueError("k_cache [blocks, kv_heads, 16, dim] and v_cache [blocks, kv_heads, vdim, 16], contiguous")
+    if block_tables.dim() != 2 or not block_tables.is_contiguous():
+        raise ValueError("block_tables must be contiguous [chunks, max_blocks]")
+    out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
+    per_channel, gs = 0, 0
+    if gate is not None:
+        per_channel = int(gate.shape[1] == num_heads * dv and dv > 1)
+        gs = _cols(gate, "gate", num_heads * dv if per_channel else num_heads)
+    ws, n = None, 0
+    if tiles is not None and num_splits > 1 and q.dtype != torch.float32:
+        n = int(num_splits)
+        ws = torch.empty(lib.mi355_softmax_bias_attn_workspace(T, num_heads, dv, n), dtype=torch.float32, device=q.device)
+    check(lib.mi355_softmax_bias_attn(
+        out.data_ptr(), q.data_ptr(), _cols(q, "q", num_heads * d), _same(k_cache, q, "k_cache"), _same(v_cache, q, "v_cache"),
+        _idx(block_tables, "block_tables", torch.int32), block_tables.shape[1], _idx(tok_seq, "tok_seq", torch.int32, T),
+        _idx(positions, "positions", torch.int64, T), None if r1 is None else _f32(r1, "r1", num_heads),
+        None if r2 is None else _f32(r2, "r2", num_heads), None if gate is None else _same(gate, q, "gate"), gs, per_channel,
+        T, num_heads, G, d, dv, int(block), int(window), float(scale),
+        None if tiles is None else _idx(tiles, "tiles", torch.int32), 0 if tiles is None else tiles.shape[0],
+        None if ws is None else ws.data_ptr(), n, dt, _stream()))
+    return out
+
+
+def mingru_scan(proj: torch.Tensor, z_off: int, x_off: int, g_off: int, channels: int, z_bias: torch.Tensor | None,
+                x_bias: torch.Tensor | None, state: torch.Tensor, cu_seqlens: torch.Tensor, positions: torch.Tensor,
+                state_slots: torch.Tensor, long_chunks: bool = True):
+    """The per-channel gated recurrence over a packed batch: proj [tokens, >= ...] holds the z, x and
+    gate projections at the given column offsets; state float32 [slots, channels] is read (unless the
+    chunk starts at position 0) and left at the chunk's last token.  Returns S * silu(gate)
+    [tokens, channels] in proj's dtype."""
+    dt = _dt3(proj, "proj")
+    T, S = proj.shape[0], cu_seqlens.numel() - 1
+    if proj.dim() != 2 or proj.stride(1) != 1:
+        raise ValueError("proj must be [tokens, columns] with a contiguous last dim")
+    if state.dim() != 2 or state.shape[1] != channels:
+        raise ValueError("state must be float32 [slots, channels]")
+    out = torch.empty(T, channels, dtype=proj.dtype, device=proj.device)
+    check(lib.mi355_mingru_scan(
+        out.data_ptr(), proj.data_ptr(), proj.stride(0) if T > 1 else proj.shape[1], int(z_off), int(x_off), int(g_off),
+        None if z_bias is None else _f32(z_bias, "z_bias", channels), None if x_bias is None else _f32(x_bias, "x_bias", channels),
+        _f32(state, "state"), _idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(positions, "positions", torch.int64, T),
+        _idx(state_slots, "state_slots", torch.int32, S), S, T, int(channels), int(bool(long_chunks)), dt, _stream()))
     return out

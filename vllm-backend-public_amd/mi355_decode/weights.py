@@ -145,6 +145,40 @@ class SandwichLayerWeights:
 
 
 @dataclass
+class MixerLayerWeights:
+    """One layer of a hybrid decoder in the "pre" arrangement whose mixer is a block attention or a
+    per-channel gated recurrence (config.BlockAttnSpec / MinGRUSpec).  Everything that reads the
+    mixer's normed input is ONE matrix in_w (segments `seg`: name -> (first column, width)):
+      attention:  q | k | g        (g: the output gate, heads * vdim wide; the values are the keys)
+      mingru:     z | x | g
+    The feed-forward is dense (up_w, down_w), a mixture of experts (router_w float32 [experts +
+    identity (+ 1), width]: the shared expert's gate row rides last in the fp32 router product;
+    expert matrices stacked [experts, ...]; the shared expert as one more gate|up and down pair), or
+    absent.  Norm weights are in the activation type, per-head numbers and biases float32."""
+    norm1: torch.Tensor
+    in_w: torch.Tensor
+    seg: dict
+    o_w: torch.Tensor
+    q_norm: Optional[torch.Tensor] = None   # f32 [dim]
+    k_norm: Optional[torch.Tensor] = None   # f32 [dim]
+    r1: Optional[torch.Tensor] = None       # f32 [heads]
+    r2: Optional[torch.Tensor] = None       # f32 [heads]
+    z_b: Optional[torch.Tensor] = None      # f32 [width of the recurrence]
+    x_b: Optional[torch.Tensor] = None
+    norm2: Optional[torch.Tensor] = None
+    up_w: Optional[torch.Tensor] = None     # dense: [ff, width]
+    down_w: Optional[torch.Tensor] = None   # dense: [width, ff]; mixture: [experts, width, ff]
+    router_w: Optional[torch.Tensor] = None
+    correction: Optional[torch.Tensor] = None   # f32 [experts + identity]
+    gate_up_w: Optional[torch.Tensor] = None    # [experts, 2 ff, width]
+    shared_gate_up_w: Optional[torch.Tensor] = None     # [2 shared_ff, width]
+    shared_down_w: Optional[torch.Tensor] = None        # [width, shared_ff]
+
+    def tensors(self):
+        return [t for t in vars(self).values() if isinstance(t, torch.Tensor)]
+
+
+@dataclass
 class ModelWeights:
     embed: torch.Tensor
     layers: list = field(default_factory=list)
@@ -155,17 +189,18 @@ class ModelWeights:
     final_norm_b: Optional[torch.Tensor] = None
     loop_step: Optional[torch.Tensor] = None     # hybrid decoders with a loop: [passes, width]
     embed_norm: Optional[torch.Tensor] = None    # hybrid decoders that norm the embedding: f32 [width]
+    bigram: Optional[torch.Tensor] = None        # hashed previous-token embedding: [buckets + 1, width]
 
     def nbytes(self) -> int:
         total = self.embed.numel() * self.embed.element_size()
         if self.lm_head.untyped_storage().data_ptr() != self.embed.untyped_storage().data_ptr():
             total += self.lm_head.numel() * self.lm_head.element_size()
         total += self.final_norm.numel() * self.final_norm.element_size()
-        for t in (self.pos_embed, self.final_norm_b, self.loop_step, self.embed_norm):
+        for t in (self.pos_embed, self.final_norm_b, self.loop_step, self.embed_norm, self.bigram):
             if t is not None:
                 total += t.numel() * t.element_size()
         for lw in self.layers:
-            ts = lw.tensors() if isinstance(lw, (OPTLayerWeights, HybridLayerWeights, SandwichLayerWeights)) else \
+            ts = lw.tensors() if isinstance(lw, (OPTLayerWeights, HybridLayerWeights, SandwichLayerWeights, MixerLayerWeights)) else \
                 (lw.qkv_w, lw.qkv_b, lw.o_w, lw.gate_up_w, lw.down_w, lw.input_norm, lw.post_norm)
             for t in ts:
                 if t is not None:
@@ -321,6 +356,8 @@ def _hybrid_from_getter(cfg: ModelConfig, get, dtype, device, tp_size: int, num_
     W = cfg.hidden_size
     if spec.arrangement == "sandwich":
         return _sandwich_from_getter(cfg, get, dtype, device)
+    if cfg.architecture == "Tafisun":
+        return _tafisun_from_getter(cfg, get, dtype, device)
 
     def put(t, dt=dtype):
         return t.to(dt).contiguous().to(device)
@@ -473,6 +510,114 @@ def _sandwich_from_getter(cfg: ModelConfig, get, dtype, device) -> ModelWeights:
     return w
 
 
+def _tafisun_from_getter(cfg: ModelConfig, get, dtype, device) -> ModelWeights:
+    """Tafisun checkpoints: 'embed', 'bigram', 'final.norm', 'head', and per layer i 'l<i>.norm1|norm2',
+    'l<i>.mix.*' (attention: q k q.norm k.norm r1 r2 g o; mingru: z z.b x x.b g o), 'l<i>.mlp.up|down'
+    (dense) or 'l<i>.mlp.router|correction', 'l<i>.mlp.e<j>.gate|up|down' and
+    'l<i>.mlp.shared.gate|up|down|sg' (mixture).  Linear weights are [out, in]."""
+    spec, W = cfg.hybrid, cfg.hidden_size
+
+    def put(t, dt=dtype):
+        return t.to(dt).contiguous().to(device)
+
+    def f32(t):
+        return put(t.reshape(-1), torch.float32)
+
+    def expect(name, shape):
+        t = get(name)
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t
+
+    w = ModelWeights(embed=put(expect("embed", (cfg.vocab_size, W))))
+    if spec.bigram is not None:
+        w.bigram = put(expect("bigram", (spec.bigram.buckets + 1, W)))
+    for i, L in enumerate(spec.layers):
+        p, m = f"l{i}.", f"l{i}.mix."
+        if L.kind == "attention":
+            A = L.battn
+            in_w, seg = _fuse_segments([("q", expect(m + "q", (A.heads * A.dim, W))), ("k", expect(m + "k", (A.kv_heads * A.dim, W))),
+                                        ("g", expect(m + "g", (A.heads * A.vdim, W)))], W, put)
+            lw = MixerLayerWeights(norm1=put(expect(p + "norm1", (W,))), in_w=in_w, seg=seg,
+                                   o_w=put(expect(m + "o", (W, A.heads * A.vdim))),
+                                   q_norm=f32(expect(m + "q.norm", (A.dim,))), k_norm=f32(expect(m + "k.norm", (A.dim,))),
+                                   r1=f32(expect(m + "r1", (A.heads,))), r2=f32(expect(m + "r2", (A.heads,))))
+        else:
+            C = L.gru.width
+            in_w, seg = _fuse_segments([(n, expect(m + n, (C, W))) for n in "zxg"], W, put)
+            lw = MixerLayerWeights(norm1=put(expect(p + "norm1", (W,))), in_w=in_w, seg=seg, o_w=put(expect(m + "o", (W, C))),
+                                   z_b=f32(expect(m + "z.b", (C,))), x_b=f32(expect(m + "x.b", (C,))))
+        q = p + "mlp."
+        if L.ff:
+            lw.norm2 = put(expect(p + "norm2", (W,)))
+            lw.up_w, lw.down_w = put(expect(q + "up", (L.ff, W))), put(expect(q + "down", (W, L.ff)))
+        elif L.moe is not None:
+            M = L.moe
+            lw.norm2 = put(expect(p + "norm2", (W,)))
+            router = [expect(q + "router", (M.outputs, W))]
+            if M.shared_ff:
+                router.append(expect(q + "shared.sg", (1, W)))
+                lw.shared_gate_up_w = put(torch.cat([expect(q + "shared.gate", (M.shared_ff, W)),
+                                                     expect(q + "shared.up", (M.shared_ff, W))], dim=0))
+                lw.shared_down_w = put(expect(q + "shared.down", (W, M.shared_ff)))
+            lw.router_w = put(torch.cat(router, dim=0), torch.float32)
+            lw.correction = f32(expect(q + "correction", (M.outputs,)))
+            lw.gate_up_w = put(torch.stack([torch.cat([expect(f"{q}e{e}.gate", (M.ff, W)), expect(f"{q}e{e}.up", (M.ff, W))],
+                                                      dim=0) for e in range(M.experts)]))
+            lw.down_w = put(torch.stack([expect(f"{q}e{e}.down", (W, M.ff)) for e in range(M.experts)]))
+        w.layers.append(lw)
+    w.final_norm = put(expect("final.norm", (W,)))
+    w.lm_head = put(expect("head", (cfg.vocab_size, W)))
+    return w
+
+
+def tafisun_synthetic_state(cfg: ModelConfig, seed: int = 0, device="cpu", dtype=torch.float32) -> dict:
+    """Seeded random tensors under a Tafisun checkpoint's names (benchmarks and tests: nothing can be
+    downloaded)."""
+    spec, W = cfg.hybrid, cfg.hidden_size
+    gen = torch.Generator(device=device).manual_seed(seed)
+
+    def mat(*shape, s=1.0):
+        return torch.empty(shape, dtype=dtype, device=device).normal_(0.0, s, generator=gen)
+
+    def near(value, *shape, s=0.1):
+        return torch.full(shape, float(value), dtype=dtype, device=device) + mat(*shape, s=s)
+
+    st = {"embed": mat(cfg.vocab_size, W), "head": mat(cfg.vocab_size, W, s=W ** -0.5), "final.norm": near(1.0, W)}
+    if spec.bigram is not None:
+        st["bigram"] = mat(spec.bigram.buckets + 1, W, s=0.5)
+    for i, L in enumerate(spec.layers):
+        p, m, q = f"l{i}.", f"l{i}.mix.", f"l{i}.mlp."
+        st[p + "norm1"] = near(1.0, W)
+        if L.kind == "attention":
+            A = L.battn
+            st[m + "q"], st[m + "k"] = mat(A.heads * A.dim, W, s=W ** -0.5), mat(A.kv_heads * A.dim, W, s=W ** -0.5)
+            st[m + "q.norm"], st[m + "k.norm"] = near(1.0, A.dim), near(1.0, A.dim)
+            st[m + "r1"], st[m + "r2"] = near(0.5, A.heads, s=0.2).abs(), near(0.3, A.heads, s=0.1).abs()
+            st[m + "g"] = mat(A.heads * A.vdim, W, s=W ** -0.5)
+            st[m + "o"] = mat(W, A.heads * A.vdim, s=(A.heads * A.vdim) ** -0.5)
+        else:
+            C = L.gru.width
+            for n in "zxg":
+                st[m + n] = mat(C, W, s=W ** -0.5)
+            st[m + "z.b"], st[m + "x.b"] = mat(C, s=0.5), mat(C, s=0.5)
+            st[m + "o"] = mat(W, C, s=C ** -0.5)
+        if L.ff:
+            st[p + "norm2"] = near(1.0, W)
+            st[q + "up"], st[q + "down"] = mat(L.ff, W, s=W ** -0.5), mat(W, L.ff, s=L.ff ** -0.5)
+        elif L.moe is not None:
+            M = L.moe
+            st[p + "norm2"] = near(1.0, W)
+            st[q + "router"], st[q + "correction"] = mat(M.outputs, W, s=W ** -0.5), mat(M.outputs, s=0.05)
+            for e in range(M.experts):
+                st[f"{q}e{e}.gate"], st[f"{q}e{e}.up"] = mat(M.ff, W, s=W ** -0.5), mat(M.ff, W, s=W ** -0.5)
+                st[f"{q}e{e}.down"] = mat(W, M.ff, s=M.ff ** -0.5)
+            if M.shared_ff:
+                st[q + "shared.gate"], st[q + "shared.up"] = mat(M.shared_ff, W, s=W ** -0.5), mat(M.shared_ff, W, s=W ** -0.5)
+                st[q + "shared.down"], st[q + "shared.sg"] = mat(W, M.shared_ff, s=M.shared_ff ** -0.5), mat(1, W, s=W ** -0.5)
+    return st
+
+
 def sandwich_synthetic_state(cfg: ModelConfig, seed: int = 0, decay_rank: int = 64, device="cpu",
                              dtype=torch.float32) -> dict:
     """Seeded random tensors under a Tativik checkpoint's names (benchmarks and tests: nothing can be
@@ -527,6 +672,8 @@ def hybrid_synthetic_state(cfg: ModelConfig, seed: int = 0, std: float = 0.02, r
     spec, W = cfg.hybrid, cfg.hidden_size
     if spec.arrangement == "sandwich":
         return sandwich_synthetic_state(cfg, seed=seed, device=device, dtype=dtype)
+    if cfg.architecture == "Tafisun":
+        return tafisun_synthetic_state(cfg, seed=seed, device=device, dtype=dtype)
     gen = torch.Generator(device=device).manual_seed(seed)
 
     def mat(*shape, s=std):

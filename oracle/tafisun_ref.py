@@ -29,8 +29,6 @@ Feed-forward
 """
 from __future__ import annotations
 
-import math
-
 import torch
 
 
@@ -70,22 +68,30 @@ def block_mask(T, size):
     return (i[None, :] <= i[:, None]) & ((i[:, None] // size) == (i[None, :] // size))
 
 
+def block_attention(q, k, wq, wk, r1, r2, scale, size, eps, gate=None):
+    """q [T, H, d], k [T, G, d] as projected.  Returns the gated, concatenated heads [T, H * d]."""
+    T, H, d = q.shape
+    G = k.shape[1]
+    v = k                                                   # the values are the keys before their norm
+    qn, kn = rms_norm(q, wq, eps), rms_norm(k, wk, eps)
+    rep = H // G
+    ke, ve = kn.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
+    s = torch.einsum("ihd,jhd->hij", qn, ke) * float(scale)
+    s = s - distance_bias(r1, r2, T, q.dtype)
+    mask = block_mask(T, size) if size else block_mask(T, T)
+    s = s.masked_fill(~mask[None], float("-inf"))
+    o = torch.einsum("hij,jhd->ihd", torch.softmax(s, dim=-1), ve).reshape(T, H * d)
+    return o if gate is None else o * torch.sigmoid(gate)
+
+
 def attention_mixer(wt, p, m, h, eps):
     H, G, d = int(m["heads"]), int(m["kv_heads"]), int(m["dim"])
     T = h.shape[0]
     q = (h @ wt[p + "q"].T).view(T, H, d)
     k = (h @ wt[p + "k"].T).view(T, G, d)
-    v = k                                                   # the values are the keys before their norm
-    qn = rms_norm(q, wt[p + "q.norm"], eps)
-    kn = rms_norm(k, wt[p + "k.norm"], eps)
-    rep = H // G
-    ke, ve = kn.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)
-    s = torch.einsum("ihd,jhd->hij", qn, ke) * float(m["scale"])
-    s = s - distance_bias(wt[p + "r1"], wt[p + "r2"], T, h.dtype)
-    s = s.masked_fill(~block_mask(T, int(m["mask"]["size"]))[None], float("-inf"))
-    a = torch.softmax(s, dim=-1)
-    o = torch.einsum("hij,jhd->ihd", a, ve).reshape(T, H * d)
-    return (o * torch.sigmoid(h @ wt[p + "g"].T)) @ wt[p + "o"].T
+    o = block_attention(q, k, wt[p + "q.norm"], wt[p + "k.norm"], wt[p + "r1"], wt[p + "r2"], m["scale"],
+                        int((m.get("mask") or {}).get("size") or 0), eps, h @ wt[p + "g"].T)
+    return o @ wt[p + "o"].T
 
 
 def mingru_candidate(u):
@@ -179,3 +185,53 @@ def forward(wt, cfg, tokens, dtype=torch.float32, trace=None):
         if trace is not None:
             trace.append(x.clone())
     return rms_norm(x, wt["final.norm"], eps) @ wt["head"].T
+
+
+def random_state(cfg, seed=0, bf16_grid=True):
+    """Seeded random tensors under the checkpoint names of `cfg` (a config dict), float32; with
+    bf16_grid every value is representable in bfloat16."""
+    g = torch.Generator().manual_seed(seed)
+    W, V = cfg["width"], cfg["vocab"]
+
+    def mat(*shape, s=1.0, mean=0.0):
+        t = torch.randn(tuple(shape), generator=g) * s + mean
+        return t.to(torch.bfloat16).float() if bf16_grid else t
+
+    st = {"embed": mat(V, W), "head": mat(V, W, s=W ** -0.5), "final.norm": mat(W, s=0.1, mean=1.0)}
+    b = (cfg.get("embedding") or {}).get("bigram")
+    if b:
+        st["bigram"] = mat(b["buckets"] + 1, W, s=0.7)
+    for i, L in enumerate(cfg["layers"]):
+        p, q, f = f"l{i}.", f"l{i}.mix.", f"l{i}.mlp."
+        st[p + "norm1"] = mat(W, s=0.1, mean=1.0)
+        m = L["mixer"]
+        if L["type"] == "attention":
+            H, G, d = m["heads"], m["kv_heads"], m["dim"]
+            st[q + "q"], st[q + "k"] = mat(H * d, W, s=W ** -0.5), mat(G * d, W, s=W ** -0.5)
+            st[q + "q.norm"], st[q + "k.norm"] = mat(d, s=0.2, mean=1.0), mat(d, s=0.2, mean=1.0)
+            st[q + "r1"], st[q + "r2"] = mat(H, s=0.4, mean=0.6).abs(), mat(H, s=0.2, mean=0.4).abs()
+            st[q + "g"], st[q + "o"] = mat(H * d, W, s=W ** -0.5), mat(W, H * d, s=(H * d) ** -0.5)
+        else:
+            C = m["width"]
+            for n in "zxg":
+                st[q + n] = mat(C, W, s=W ** -0.5)
+            st[q + "z.b"], st[q + "x.b"] = mat(C, s=0.7), mat(C, s=0.7)
+            st[q + "o"] = mat(W, C, s=C ** -0.5)
+        mlp = L.get("mlp")
+        if mlp is None:
+            continue
+        st[p + "norm2"] = mat(W, s=0.1, mean=1.0)
+        if mlp.get("kind", "dense") == "dense":
+            st[f + "up"], st[f + "down"] = mat(mlp["ff"], W, s=W ** -0.5), mat(W, mlp["ff"], s=mlp["ff"] ** -0.5)
+            continue
+        r, F = mlp["router"], mlp["expert"]["ff"]
+        n = r["experts"] + r.get("identity", 0)
+        st[f + "router"], st[f + "correction"] = mat(n, W, s=2.0 * W ** -0.5), mat(n, s=0.1)
+        for e in range(r["experts"]):
+            st[f"{f}e{e}.gate"], st[f"{f}e{e}.up"] = mat(F, W, s=2.0 * W ** -0.5), mat(F, W, s=2.0 * W ** -0.5)
+            st[f"{f}e{e}.down"] = mat(W, F, s=F ** -0.5)
+        if mlp.get("shared"):
+            S = mlp["shared"]["ff"]
+            st[f + "shared.gate"], st[f + "shared.up"] = mat(S, W, s=2.0 * W ** -0.5), mat(S, W, s=2.0 * W ** -0.5)
+            st[f + "shared.down"], st[f + "shared.sg"] = mat(W, S, s=S ** -0.5), mat(1, W, s=W ** -0.5)
+    return st

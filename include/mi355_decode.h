@@ -1009,7 +1009,10 @@ int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const fl
  *   mingru_scan           S <- (1 - z) S + z c per channel, z = sigmoid(zp + z_bias), u = xp + x_bias,
  *                         c = u + 1/2 (u >= 0) or sigmoid(u); out = S * silu(gp); zp / xp / gp are the
  *                         column ranges z_off / x_off / g_off of the projection rows; state fp32
- *                         [slots, channels], reset by a chunk that starts at position 0
+ *                         [slots, channels], reset by a chunk that starts at position 0.  long_chunks:
+ *                         some chunk holds several rows (16 waves per workgroup share a chunk); with
+ *                         num_parts > 1 and a workspace (mingru_scan_workspace floats) every chunk is
+ *                         also dealt out to that many workgroups, in two launches
  */
 int32_t mi355_embed_bigram_pos_f32(float* out, const void* embed, const void* bigram, const int64_t* ids,
                                    const int64_t* positions, const int32_t* cu_seqlens,
@@ -1039,7 +1042,9 @@ int32_t mi355_mingru_scan(void* out, const void* proj, int64_t stride, int32_t z
                           int32_t g_off, const float* z_bias, const float* x_bias, float* state,
                           const int32_t* cu_seqlens, const int64_t* positions,
                           const int32_t* state_slots, int32_t num_seqs, int64_t num_tokens,
-                          int32_t channels, int32_t long_chunks, int32_t dtype, void* stream);
+                          int32_t channels, int32_t long_chunks, float* workspace, int32_t num_parts,
+                          int32_t dtype, void* stream);
+int64_t mi355_mingru_scan_workspace(int32_t num_seqs, int32_t channels, int32_t num_parts);
 
 #ifdef __cplusplus
 }

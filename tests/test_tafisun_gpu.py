@@ -294,7 +294,7 @@ def test_distance_penalty_moves_weight_to_near_keys():
     assert abs(float(got[-1, 0]) - (T + 1) / 2) < 1e-3 and abs(float(got[-1, d]) - want1) < 1e-3
 
 
-def _gru_in_steps(x, bz, bx, C, chunks_per_step, state):
+def _gru_in_steps(x, bz, bx, C, chunks_per_step, state, parts=None):
     """x [T, 3 C + pad] rows of one or more sequences; chunks_per_step: [[(row slice, first position, slot)]]."""
     from mi355_decode import ops
     outs = {}
@@ -302,7 +302,8 @@ def _gru_in_steps(x, bz, bx, C, chunks_per_step, state):
         rows = torch.cat([x[c[0]] for c in chunks]).contiguous().cuda()
         pos = torch.cat([torch.arange(c[1], c[1] + (c[0].stop - c[0].start)) for c in chunks]).cuda()
         out = ops.mingru_scan(rows, 8, 8 + C, 8 + 2 * C, C, bz.cuda(), bx.cuda(), state, _cu([c[0].stop - c[0].start for c in chunks]),
-                              pos, _i32([c[2] for c in chunks]), long_chunks=max(c[0].stop - c[0].start for c in chunks) > 1)
+                              pos, _i32([c[2] for c in chunks]), long_chunks=max(c[0].stop - c[0].start for c in chunks) > 1,
+                              num_parts=parts)
         at = 0
         for c in chunks:
             n = c[0].stop - c[0].start
@@ -331,12 +332,13 @@ def test_mingru_whole_portions_single_tokens_and_long_prompts(dtype, C):
     state = torch.full((3, C), float("nan"), device="cuda")
     cuts_list = [[T], [2, 3, 1, 30, 2, 16, T - 54]] + ([[1] * T] if T < 200 else [[700, 1, 799]])
     for cuts in cuts_list:
-        steps, at = [], 0
-        for n in cuts:
-            steps.append([(slice(at, at + n), at, 1)])
-            at += n
-        got = _gru_in_steps(x, bz, bx, C, steps, state)[1]
-        assert (got - ref).abs().max() <= tol * ref.abs().max(), cuts
+        for parts in (None, 1, 3, 16):                         # a chunk dealt out to several workgroups, two launches
+            steps, at = [], 0
+            for n in cuts:
+                steps.append([(slice(at, at + n), at, 1)])
+                at += n
+            got = _gru_in_steps(x, bz, bx, C, steps, state, parts)[1]
+            assert (got - ref).abs().max() <= tol * ref.abs().max(), (cuts, parts)
 
 
 def test_mingru_slots_are_separate_reset_at_position_zero_and_hold_a_value():

@@ -35,7 +35,7 @@ __global__ __launch_bounds__(256) void qk_norm_kv_write_kernel(
     const int g = h - H;
     if (!is_q && slot < 0) continue;
     const E* src = is_q ? q + t * q_stride + static_cast<int64_t>(h) * d : k + t * k_stride + static_cast<int64_t>(g) * d;
-    const void* base = is_q ? static_cast<const void*>(q) : static_cast<const void*>(k);
+    [[maybe_unused]] const void* base = is_q ? static_cast<const void*>(q) : static_cast<const void*>(k);
     float ss = 0.f;
     for (int i = lane; i < d; i += 64) {
       const float x = MI355_LDF(T, base, src + i);

@@ -286,14 +286,17 @@ __global__ __launch_bounds__(256) void embed_bigram_pos_f32_kernel(
     brow = bigram + row * W;
   }
   const float pf = static_cast<float>(p);
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    float v = MI355_LDF(T, embed, embed + id * W + c);
-    if (brow != nullptr) v += MI355_LDF(T, bigram, brow + c);
-    if (freq != nullptr) {
-      const float a = pf * MI355_LD(float, freq, freq + (c >> 1));
-      v += (c & 1) ? cosf(a) : sinf(a);
+  for (int i = threadIdx.x; 2 * i < W; i += blockDim.x) {     // a pair of columns shares its angle
+    float sn = 0.f, cs = 0.f;
+    if (freq != nullptr) sincosf(pf * MI355_LD(float, freq, freq + i), &sn, &cs);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int c = 2 * i + j;
+      if (c >= W) break;
+      float v = MI355_LDF(T, embed, embed + id * W + c);
+      if (brow != nullptr) v += MI355_LDF(T, bigram, brow + c);
+      MI355_ST(float, out, out + t * W + c, v + (j ? cs : sn));
     }
-    MI355_ST(float, out, out + t * W + c, v);
   }
 }
 

@@ -824,23 +824,31 @@ __global__ __launch_bounds__(64) void general_delta_rule_cols_kernel(
 }
 
 // A gated recurrence per channel whose gates read only the current token (zp, xp, gp: three column
-// ranges of the projection rows).  One workgroup per (64 channels, chunk); its waves take consecutive
-// segments of the chunk's rows.  The recurrence is linear in S, so a segment is summarised by
-// (A, B) with S_end = A S_start + B: every wave scans its segment from zero for (A, B), the
-// summaries of the earlier segments give its true start, and a second scan writes the outputs.  A
-// single wave (decoded tokens) scans once.  State, gates and candidates are fp32.
-template <typename T>
+// ranges of the projection rows).  One workgroup per (64 channels, chunk, part of the chunk); its
+// waves take consecutive segments of the part's rows.  The recurrence is linear in S, so a run of
+// rows is summarised by (A, B) with S_end = A S_start + B: every wave scans its segment from zero for
+// (A, B), the summaries of the earlier segments give its true start, and a second scan writes the
+// outputs.  A single wave (decoded tokens) scans once.  With several parts per chunk (gridDim.z > 1:
+// long prompts, few chunks) a first launch (PASS 1) leaves every part's summary in `parts`
+// [chunks, parts, channels, 2], and the second (PASS 2) starts every part from the summaries of
+// the parts before it.  State, gates and candidates are fp32.
+template <typename T, int PASS>
 __global__ __launch_bounds__(1024) void mingru_scan_kernel(
     typename Elem<T>::S* __restrict__ out, const typename Elem<T>::S* __restrict__ proj, int64_t stride, int z_off, int x_off,
     int g_off, const float* __restrict__ bz, const float* __restrict__ bx, float* __restrict__ state,
     const int32_t* __restrict__ cu_seqlens, const int64_t* __restrict__ positions, const int32_t* __restrict__ state_slots,
-    int C) {
+    int C, float* __restrict__ parts) {
   __shared__ float sa[16][64], sb[16][64];
   const int s = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
   const int c = blockIdx.x * 64 + lane;
   const bool live = c < C;
-  const int r0 = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s), r1 = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s + 1);
-  if (r1 <= r0) return;                                 // (the whole workgroup)
+  const int q0 = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s), q1 = MI355_LD(int32_t, cu_seqlens, cu_seqlens + s + 1);
+  if (q1 <= q0) return;                                 // (the whole workgroup)
+  // this workgroup's part of the chunk
+  const int nz = gridDim.z, zi = blockIdx.z;
+  const int per_z = (q1 - q0 + nz - 1) / nz;
+  const int r0 = q0 + zi * per_z < q1 ? q0 + zi * per_z : q1;
+  const int r1 = r0 + per_z < q1 ? r0 + per_z : q1;
   const int per = (r1 - r0 + nw - 1) / nw;
   const int a = r0 + wave * per < r1 ? r0 + wave * per : r1;
   const int b = a + per < r1 ? a + per : r1;
@@ -852,7 +860,7 @@ __global__ __launch_bounds__(1024) void mingru_scan_kernel(
     const float u = MI355_LDF(T, proj, row + x_off + c) + xb;
     cand = u >= 0.f ? u + 0.5f : 1.0f / (1.0f + expf(-u));
   };
-  if (nw > 1) {
+  if (nw > 1 || PASS == 1) {
     float A = 1.0f, B = 0.f;
     if (live) {
       for (int t = a; t < b; ++t) {
@@ -866,9 +874,28 @@ __global__ __launch_bounds__(1024) void mingru_scan_kernel(
     sb[wave][lane] = B;
     __syncthreads();
   }
+  if (PASS == 1) {                                      // the part's summary: its waves' summaries in turn
+    if (wave == 0 && live) {
+      float A = 1.0f, B = 0.f;
+      for (int i = 0; i < nw; ++i) {
+        B = sa[i][lane] * B + sb[i][lane];
+        A *= sa[i][lane];
+      }
+      float* dst = parts + ((static_cast<int64_t>(s) * nz + zi) * C + c) * 2;
+      MI355_ST(float, parts, dst, A);
+      MI355_ST(float, parts, dst + 1, B);
+    }
+    return;
+  }
   if (!live || a >= b) return;
   const int64_t slot = MI355_LD(int32_t, state_slots, state_slots + s);
-  float S = MI355_LD(int64_t, positions, positions + r0) > 0 ? MI355_LD(float, state, state + slot * C + c) : 0.f;
+  float S = MI355_LD(int64_t, positions, positions + q0) > 0 ? MI355_LD(float, state, state + slot * C + c) : 0.f;
+  if (PASS == 2) {
+    for (int i = 0; i < zi; ++i) {
+      const float* src = parts + ((static_cast<int64_t>(s) * nz + i) * C + c) * 2;
+      S = MI355_LD(float, parts, src) * S + MI355_LD(float, parts, src + 1);
+    }
+  }
   for (int i = 0; i < wave; ++i) S = sa[i][lane] * S + sb[i][lane];
   for (int t = a; t < b; ++t) {
     float z, cand;
@@ -877,7 +904,7 @@ __global__ __launch_bounds__(1024) void mingru_scan_kernel(
     const float g = MI355_LDF(T, proj, proj + static_cast<int64_t>(t) * stride + g_off + c);
     MI355_STF(T, out, out + static_cast<int64_t>(t) * C + c, S * (g / (1.0f + expf(-g))));
   }
-  if (b == r1) MI355_ST(float, state, state + slot * C + c, S);
+  if (b == q1) MI355_ST(float, state, state + slot * C + c, S);
 }
 
 // out = sigmoid(gate) * sum of the key-range partial sums of sigmoid_window_attn_mfma_kernel
@@ -1221,24 +1248,40 @@ extern "C" int32_t mi355_general_delta_rule(float* o, const void* r, int64_t r_s
   return check_launch("general_delta_rule");
 }
 
+extern "C" int64_t mi355_mingru_scan_workspace(int32_t num_seqs, int32_t channels, int32_t num_parts) {
+  return num_parts > 1 ? static_cast<int64_t>(num_seqs) * num_parts * channels * 2 : 0;          // floats
+}
+
 extern "C" int32_t mi355_mingru_scan(void* out, const void* proj, int64_t stride, int32_t z_off, int32_t x_off, int32_t g_off,
                                      const float* z_bias, const float* x_bias, float* state, const int32_t* cu_seqlens,
                                      const int64_t* positions, const int32_t* state_slots, int32_t num_seqs,
-                                     int64_t num_tokens, int32_t channels, int32_t long_chunks, int32_t dtype, void* stream) {
+                                     int64_t num_tokens, int32_t channels, int32_t long_chunks, float* workspace,
+                                     int32_t num_parts, int32_t dtype, void* stream) {
   MI355_REQUIRE(out && proj && state && cu_seqlens && positions && state_slots, MI355_ERR_INVALID, "mingru_scan: null pointer");
   MI355_REQUIRE(num_seqs >= 0 && num_seqs <= 65535 && num_tokens >= 0 && channels > 0 && z_off >= 0 && x_off >= 0 && g_off >= 0,
                 MI355_ERR_INVALID, "mingru_scan: sizes");
   MI355_REQUIRE(stride >= static_cast<int64_t>(z_off) + channels && stride >= static_cast<int64_t>(x_off) + channels &&
                     stride >= static_cast<int64_t>(g_off) + channels,
                 MI355_ERR_INVALID, "mingru_scan: rows shorter than the column ranges");
+  MI355_REQUIRE(num_parts >= 0 && num_parts <= 64 && (num_parts <= 1 || workspace != nullptr), MI355_ERR_INVALID,
+                "mingru_scan: %d parts per chunk need a workspace", num_parts);
   REQ_DTYPE(dtype);
   if (num_tokens == 0 || num_seqs == 0) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>((channels + 63) / 64), static_cast<unsigned>(num_seqs));
+  const unsigned nz = (long_chunks && num_parts > 1) ? static_cast<unsigned>(num_parts) : 1u;
+  const dim3 grid(static_cast<unsigned>((channels + 63) / 64), static_cast<unsigned>(num_seqs), nz);
   const dim3 block(long_chunks ? 1024 : 64);
-  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((mingru_scan_kernel<TT>), grid, block, 0, s,
-                                                  static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(proj), stride,
-                                                  z_off, x_off, g_off, z_bias, x_bias, state, cu_seqlens, positions,
-                                                  state_slots, channels));
+#define MI355_GRU(PASS)                                                                                                  \
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((mingru_scan_kernel<TT, PASS>), grid, block, 0, s,                     \
+                                                  static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(proj), \
+                                                  stride, z_off, x_off, g_off, z_bias, x_bias, state, cu_seqlens,        \
+                                                  positions, state_slots, channels, workspace))
+  if (nz > 1) {
+    MI355_GRU(1);
+    MI355_GRU(2);
+  } else {
+    MI355_GRU(0);
+  }
+#undef MI355_GRU
   return check_launch("mingru_scan");
 }

@@ -139,7 +139,8 @@ def _load() -> ctypes.CDLL:
         "mi355_softmax_bias_attn_workspace": (I64, [I64, I32, I32, I32]),
         "mi355_softmax_bias_attn": (I32, [P, P, I64, P, P, P, I32, P, P, P, P, P, I64, I32, I64, I32, I32, I32, I32, I32,
                                           I32, F, P, I32, P, I32, I32, P]),
-        "mi355_mingru_scan": (I32, [P, P, I64, I32, I32, I32, P, P, P, P, P, P, I32, I64, I32, I32, I32, P]),
+        "mi355_mingru_scan": (I32, [P, P, I64, I32, I32, I32, P, P, P, P, P, P, I32, I64, I32, I32, P, I32, I32, P]),
+        "mi355_mingru_scan_workspace": (I64, [I32, I32, I32]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)          # AttributeError if the symbol is missing
@@ -180,7 +181,8 @@ EXPORTS = ("mi355_abi_version", "mi355_last_error", "mi355_target_arch",
            "mi355_latent_window_attn", "mi355_moe_route", "mi355_moe_sort", "mi355_moe_gather_rows",
            "mi355_moe_gate_up_rows", "mi355_moe_down_rows", "mi355_moe_silu_and_mul", "mi355_moe_combine",
            "mi355_embed_bigram_pos_f32", "mi355_prev_token_update", "mi355_relu_squared", "mi355_qk_norm_kv_write",
-           "mi355_softmax_bias_attn_workspace", "mi355_softmax_bias_attn", "mi355_mingru_scan")
+           "mi355_softmax_bias_attn_workspace", "mi355_softmax_bias_attn", "mi355_mingru_scan",
+           "mi355_mingru_scan_workspace")
 
 
 def check(status: int) -> None:

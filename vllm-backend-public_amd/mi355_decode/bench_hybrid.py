@@ -44,6 +44,21 @@ def tativik_config(width: int, layers: int, vocab: int = 32000) -> dict:
             "residual_mult": 0.7, "layers": ls}
 
 
+def tafisun_config(width: int, layers: int, vocab: int = 32000) -> dict:
+    """Alternating block-attention / minGRU layers: 128-wide heads, four query heads to a key head,
+    blocks of 1024 positions; a recurrence as wide as the model; a dense relu^2 feed-forward of
+    2 * width in the first layer and, in the others, 30 experts + 2 identity outputs of width / 2
+    with 4 per token out of 2 of 4 groups, beside a shared expert of width / 2."""
+    nh = width // 128
+    att = {"heads": nh, "kv_heads": max(nh // 4, 1), "dim": 128, "vdim": 128, "mask": {"size": 1024}, "scale": 128 ** -0.5}
+    moe = {"kind": "moe", "expert": {"ff": width // 2, "limit": 7.0}, "shared": {"ff": width // 2, "limit": 7.0},
+           "router": {"experts": 30, "identity": 2, "top": 4, "scale": 1.5, "groups": {"count": 4, "keep": 2}}}
+    ls = [{"type": "attention" if i % 2 == 0 else "mingru", "mixer": att if i % 2 == 0 else {"width": width},
+           "mlp": {"kind": "dense", "ff": 2 * width} if i == 0 else moe} for i in range(layers)]
+    return {"architecture": "Tafisun", "width": width, "vocab": vocab, "norm": {"eps": 1e-6},
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 7919}}, "layers": ls}
+
+
 def lozupel_config(width: int, layers: int, vocab: int = 32000, loop: bool = True) -> dict:
     """Alternating parallel / delta layers with 128-wide heads, a 1024-token window, a feed-forward in
     every layer; the middle of the stack loops twice."""
@@ -397,4 +412,155 @@ def compare_tativik(widths, layers: int, batch: int, prompt_len: int, steps: int
                                  "prefill_ratio": round(t["prefill_tok_s"] / z["prefill_tok_s"], 3),
                                  "decode_ratio": round(t["decode_tok_s"] / z["decode_tok_s"], 3)})
         result["kernels"][str(width)] = tativik_kernel_table(width, prompt_len, batch)
+    return result
+
+
+def tafisun_kernel_table(width: int, prompt_len: int, batch: int) -> list:
+    """The Tafisun design's kernels at the prefill and the decode shape, each against its own
+    roofline, beside the like kernel of the closest existing designs at the same shape."""
+    from types import SimpleNamespace
+    from .config import MoESpec
+    from .hybrid_runner import MoEFeedForward
+    dev, bf = "cuda", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rnd = lambda *s, dt=bf: torch.randn(*s, device=dev, dtype=torch.float32, generator=g).to(dt)  # noqa: E731
+    rows = []
+
+    def row(kernel, shape, t, bound, work, like=None, like_t=None, like_work=None, like_bound=None):
+        peak = {"hbm": HBM, "mfma": MFMA, "valu": VALU}
+        r = {"kernel": kernel, "shape": shape, "us": round(t * 1e6, 2), "bound": bound,
+             "frac_of_roofline": round(work / peak[bound] / t, 4)}
+        if like is not None:
+            r.update(like=like, like_us=round(like_t * 1e6, 2), like_frac=round(like_work / peak[like_bound or bound] / like_t, 4))
+            r["distance_ratio"] = round(r["like_frac"] / max(r["frac_of_roofline"], 1e-9), 2)
+        rows.append(r)
+
+    P, W, V = prompt_len, width, 32000
+    H, G, d, block = W // 128, max(W // 512, 1), 128, 1024
+    pages = (P + BLOCK_SIZE) // BLOCK_SIZE + 1
+    nb = pages * batch
+    kc, vct = rnd(nb, G, BLOCK_SIZE, d), rnd(nb, G, d, BLOCK_SIZE)
+    bt = torch.arange(nb, dtype=torch.int32, device=dev).view(batch, pages)
+    embed, bigram = rnd(V, W), rnd(65522, W)
+    freq = torch.from_numpy((10000.0 ** (-2.0 * np.arange(W // 2) / W)).astype(np.float32)).to(dev)
+    r1, r2 = torch.full((H,), 0.5, device=dev), torch.full((H,), 0.3, device=dev)
+    temp, bias = torch.ones(H, device=dev), torch.full((H,), -2.0, device=dev)
+    wn = torch.ones(d, device=dev)
+    cs = None
+    for T, S, tag in ((P, 1, "prefill"), (batch, batch, "decode")):
+        shape = f"{tag} {T} rows x {W}"
+        per = T // S
+        cu = torch.arange(0, T + 1, per, dtype=torch.int32, device=dev)
+        pos = (torch.arange(T, device=dev) % per + (0 if S == 1 else P - 1)).to(torch.int64)
+        seq = (torch.arange(T, device=dev) // per).to(torch.int32)
+        slots = torch.arange(S, dtype=torch.int32, device=dev)
+        ids = torch.randint(0, V, (T,), device=dev, generator=g)
+        prev = torch.zeros(S + 1, dtype=torch.int32, device=dev)
+        # ---- embedding
+        row("embed_bigram_pos_f32 + prev_token_update", shape,
+            _time(lambda: (ops.embed_bigram_pos_f32(embed, ids, pos, bigram, (65521, 1000003, 7919), cu, seq, slots, prev, freq),
+                           ops.prev_token_update(prev, ids, cu, slots))), "hbm", T * W * 8,
+            "embed_scale_f32", _time(lambda: ops.embed_scale_f32(embed, ids, 1.0)), T * W * 6)
+        # ---- feed-forward activation
+        F = 2 * W
+        up, gu, act = rnd(T, F), rnd(T, 2 * F), torch.empty(T, F, device=dev, dtype=bf)
+        row("relu_squared", f"{tag} {T} rows x {F}", _time(lambda: ops.relu_squared(up)), "hbm", T * F * 4,
+            "gelu_tanh_and_mul", _time(lambda: ops.gelu_tanh_and_mul(gu, out=act)), T * F * 6)
+        # ---- attention
+        if cs is None:
+            from .hybrid_runner import rotary_table
+            cs = rotary_table(64, 1.0e6, pages * BLOCK_SIZE, dev)
+        proj = rnd(T, (2 * H + G) * d)
+        q, k, gt = proj[:, : H * d], proj[:, H * d: (H + G) * d], proj[:, (H + G) * d:]
+        v_, gh = rnd(T, G * d), rnd(T, H)
+        wslots = (torch.arange(T, device=dev) if S == 1 else torch.arange(T, device=dev) * pages * BLOCK_SIZE + P - 1).to(torch.int64)
+        row("qk_norm_kv_write", f"{tag} {T} rows, {H}/{G} heads x {d}",
+            _time(lambda: ops.qk_norm_kv_write(q, k, k, wn, wn, wslots, kc, vct, H, G, d, d, 1e-6)), "hbm",
+            T * (2 * H * d + 3 * G * d) * 2,
+            "rope_partial_kv_write", _time(lambda: ops.rope_partial_kv_write(q, k, v_, cs, pos, wslots, kc, vct, H, G, d, d)),
+            T * (2 * H * d + 4 * G * d) * 2)
+        if S == 1:
+            tiles = torch.from_numpy(ops.query_tiles([0, P])).to(dev)
+            b_t = bt[:1]
+        else:
+            tiles = torch.stack([seq, seq, torch.ones_like(seq)], dim=1).contiguous()
+            b_t = bt
+        rep = H // G
+        hb = 4 if rep % 4 == 0 else 3 if rep % 3 == 0 else 2 if rep % 2 == 0 else 1
+        nsb = max(min(16, block // 64, 2048 // max(int(tiles.shape[0]) * G * (rep // hb), 1)), 1)
+        nsw = max(min(16, 2048 // max(int(tiles.shape[0]) * G * max(rep // 4, 1), 1)), 1)
+        part = torch.empty(nsw * T * H * d, device=dev)
+        o = torch.empty(T, H * d, device=dev, dtype=bf)
+        t_n = _time(lambda: ops.softmax_bias_attn(q, kc, vct, b_t, seq, pos, r1, r2, gt, H, d ** -0.5, block=block, tiles=tiles,
+                                                  num_splits=nsb if nsb > 1 else 0), 5)
+        t_l = _time(lambda: ops.sigmoid_window_attn(q, kc, vct, b_t, seq, pos, temp, bias, gh, H, block, d ** -0.5, out=o,
+                                                    tiles=tiles, partial=part, num_splits=nsw), 5)
+        if S == 1:
+            keys_b = sum(i % block + 1 for i in range(P))
+            keys_w = sum(min(i + 1, block) for i in range(P))
+            row("softmax_bias_attn", f"prefill {P} tokens, blocks of {block}, {H}/{G} heads x {d}", t_n, "mfma",
+                2.0 * keys_b * H * 2 * d, f"sigmoid_window_attn, window {block}", t_l, 2.0 * keys_w * H * 2 * d)
+        else:
+            kb = (P - 1) % block + 1
+            row("softmax_bias_attn", f"decode {T} rows at position {P - 1}: {kb} keys each, blocks of {block}", t_n, "hbm",
+                T * kb * G * 2 * d * 2, f"sigmoid_window_attn, window {block}: {min(P, block)} keys each", t_l,
+                T * min(P, block) * G * 2 * d * 2)
+        # ---- the recurrence
+        C = W
+        x3 = rnd(T, 3 * C)
+        bz, bx = torch.zeros(C, device=dev), torch.zeros(C, device=dev)
+        st = torch.zeros(S + 1, C, device=dev)
+        t_n = _time(lambda: ops.mingru_scan(x3, 0, C, 2 * C, C, bz, bx, st, cu, pos, slots, long_chunks=S == 1), 5)
+        Hd, Gd, dd = W // 128, max(W // 256, 1), 128
+        Cd = 2 * Gd * dd + Hd * dd
+        xd, beta, dec = rnd(T, Cd), rnd(T, Hd), rnd(T, Hd)
+        a_log, dtb = torch.zeros(Hd, device=dev), torch.zeros(Hd, device=dev)
+        std = torch.zeros(S + 1, Hd, dd, dd, device=dev)
+        od = torch.empty(T, Hd, dd, device=dev)
+        t_l = _time(lambda: ops.gated_delta_rule(xd, 0, Gd * dd, 2 * Gd * dd, beta, dec, a_log, dtb, std, cu, pos, slots, Hd, Gd, dd,
+                                                 dd, out=od, long_chunks=S == 1), 5)
+        if S == 1:
+            row("mingru_scan", f"prefill {T} tokens x {C} channels", t_n, "hbm", T * C * 8,
+                f"gated_delta_rule, {Hd} heads x {dd} x {dd}", t_l, 6.0 * T * Hd * dd * dd, "valu")
+        else:
+            row("mingru_scan", f"decode {S} rows x {C} channels", t_n, "hbm", S * C * 16,
+                f"gated_delta_rule, {Hd} heads x {dd} x {dd}", t_l, S * Hd * dd * dd * 8)
+    # ---- the mixture of experts beside the sigmoid-routed one without identity and shared experts
+    E, I, top, F = 30, 2, 4, W // 2
+    lw = SimpleNamespace(router_w=rnd(E + I + 1, W, dt=torch.float32) * W ** -0.5, correction=torch.zeros(E + I, device=dev),
+                         gate_up_w=rnd(E, 2 * F, W) * W ** -0.5, down_w=rnd(E, W, F) * F ** -0.5,
+                         shared_gate_up_w=rnd(2 * F, W) * W ** -0.5, shared_down_w=rnd(W, F) * F ** -0.5)
+    lin = SimpleNamespace(linear=lambda x, w: ops.linear_decode(x, w) if x.shape[0] <= ops.LINEAR_DECODE_MAX_M else torch.mm(x, w.t()))
+    ff = MoEFeedForward(MoESpec(E, top, 4, 2, F, score="softmax", group_score="max", weight_scale=1.5, identity=I, limit=7.0,
+                                shared_ff=F, shared_limit=7.0), lw, lin)
+    lw0 = SimpleNamespace(router_w=rnd(E + I, W, dt=torch.float32) * W ** -0.5, correction=torch.zeros(E + I, device=dev),
+                          gate_up_w=rnd(E + I, 2 * F, W) * W ** -0.5, down_w=rnd(E + I, W, F) * F ** -0.5)
+    ff0 = MoEFeedForward(MoESpec(E + I, top, 4, 2, F), lw0, None)
+    for T, tag in ((P, "prefill"), (batch, "decode")):
+        h = rnd(T, W)
+        t_n, t_l = _time(lambda: ff(h), 5), _time(lambda: ff0(h), 5)
+        if tag == "prefill":
+            row("mixture (softmax route, identity, limits, shared expert)", f"prefill {T} rows, {top} of {E}+{I} x {F}, shared {F}", t_n,
+                "mfma", 6.0 * T * (top + 1) * F * W, "mixture (sigmoid route), no shared expert", t_l, 6.0 * T * top * F * W)
+        else:
+            touched = min(E, T * top)
+            row("mixture (softmax route, identity, limits, shared expert)", f"decode {T} rows, {top} of {E}+{I} x {F}, shared {F}", t_n,
+                "hbm", (touched + 1) * 3 * F * W * 2, "mixture (sigmoid route), no shared expert", t_l,
+                min(E + I, T * top) * 3 * F * W * 2)
+    return rows
+
+
+def compare_tafisun(widths, layers: int, batch: int, prompt_len: int, steps: int, warmup: int) -> dict:
+    """The Tafisun design beside the closest existing model, the sandwich arrangement (Tativik: a
+    softmax attention in a window, a recurrence, a grouped mixture of experts), at equal width and depth."""
+    result = {"metric": "tafisun_vs_tativik_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+              "config": {"layers": layers, "batch": batch, "prompt_len": prompt_len, "decode_steps": steps},
+              "models": [], "kernels": {}}
+    for width in widths:
+        t = through_engine(ModelConfig.from_dict(tafisun_config(width, layers)), batch, prompt_len, steps, warmup)
+        z = through_engine(ModelConfig.from_dict(tativik_config(width, layers)), batch, prompt_len, steps, warmup)
+        result["models"].append({"width": width, "layers": layers, "tafisun": t, "tativik": z,
+                                 "prefill_ratio": round(t["prefill_tok_s"] / z["prefill_tok_s"], 3),
+                                 "decode_ratio": round(t["decode_tok_s"] / z["decode_tok_s"], 3)})
+        result["kernels"][str(width)] = tafisun_kernel_table(width, prompt_len, batch)
     return result

@@ -1627,11 +1627,12 @@ def softmax_bias_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
 
 def mingru_scan(proj: torch.Tensor, z_off: int, x_off: int, g_off: int, channels: int, z_bias: torch.Tensor | None,
                 x_bias: torch.Tensor | None, state: torch.Tensor, cu_seqlens: torch.Tensor, positions: torch.Tensor,
-                state_slots: torch.Tensor, long_chunks: bool = True):
+                state_slots: torch.Tensor, long_chunks: bool = True, num_parts: int | None = None):
     """The per-channel gated recurrence over a packed batch: proj [tokens, >= ...] holds the z, x and
     gate projections at the given column offsets; state float32 [slots, channels] is read (unless the
-    chunk starts at position 0) and left at the chunk's last token.  Returns S * silu(gate)
-    [tokens, channels] in proj's dtype."""
+    chunk starts at position 0) and left at the chunk's last token.  long_chunks: some chunk holds
+    several rows.  num_parts: workgroups a chunk is dealt out to (None: enough to fill the chip when
+    the step has few, long chunks).  Returns S * silu(gate) [tokens, channels] in proj's dtype."""
     dt = _dt3(proj, "proj")
     T, S = proj.shape[0], cu_seqlens.numel() - 1
     if proj.dim() != 2 or proj.stride(1) != 1:
@@ -1639,9 +1640,15 @@ def mingru_scan(proj: torch.Tensor, z_off: int, x_off: int, g_off: int, channels
     if state.dim() != 2 or state.shape[1] != channels:
         raise ValueError("state must be float32 [slots, channels]")
     out = torch.empty(T, channels, dtype=proj.dtype, device=proj.device)
+    if num_parts is None:                                      # about 16 rows per wave at least, about 512 workgroups at most
+        num_parts = min(16, max(T // max(S, 1) // 256, 1), max(512 // max(S * ((channels + 63) // 64), 1), 1))
+    num_parts = int(num_parts) if long_chunks else 1
+    ws = torch.empty(lib.mi355_mingru_scan_workspace(S, channels, num_parts), dtype=torch.float32, device=proj.device) \
+        if num_parts > 1 else None
     check(lib.mi355_mingru_scan(
         out.data_ptr(), proj.data_ptr(), proj.stride(0) if T > 1 else proj.shape[1], int(z_off), int(x_off), int(g_off),
         None if z_bias is None else _f32(z_bias, "z_bias", channels), None if x_bias is None else _f32(x_bias, "x_bias", channels),
         _f32(state, "state"), _idx(cu_seqlens, "cu_seqlens", torch.int32), _idx(positions, "positions", torch.int64, T),
-        _idx(state_slots, "state_slots", torch.int32, S), S, T, int(channels), int(bool(long_chunks)), dt, _stream()))
+        _idx(state_slots, "state_slots", torch.int32, S), S, T, int(channels), int(bool(long_chunks)),
+        None if ws is None else ws.data_ptr(), num_parts, dt, _stream()))
     return out

@@ -196,14 +196,27 @@ __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
 #pragma unroll
     for (int c = 0; c < CB; ++c) acc[i][c] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  for (int64_t base = ((lo0 >> 5) << 5) + 32 * z; base <= p_last; base += 32 * nz) {
+  // the pages of a tile are looked up one tile ahead: the table's trip to memory then runs beside the
+  // current tile's K/V loads instead of in front of the next tile's
+  const int64_t first = ((lo0 >> 5) << 5) + 32 * z;
+  int32_t pg[2] = {0, 0};
+#pragma unroll
+  for (int half = 0; half < 2; ++half)
+    if (first + 16 * half <= p_last) pg[half] = MI355_LD(int32_t, block_tables, bt + (first + 16 * half) / kPageB);
+  for (int64_t base = first; base <= p_last; base += 32 * nz) {
     uint4 kf[2][DS];
     uint2 vf[2][CB];
+    int32_t npg[2] = {0, 0};
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int64_t nb = base + 32 * nz + 16 * half;
+      if (nb <= p_last) npg[half] = MI355_LD(int32_t, block_tables, bt + nb / kPageB);
+    }
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       const int64_t kb = base + 16 * half;
       const bool have = kb <= p_last;
-      const int64_t page = have ? MI355_LD(int32_t, block_tables, bt + kb / kPageB) : 0;
+      const int64_t page = pg[half];
       const uint16_t* kr = k_cache + ((page * G + g) * kPageB + li) * d + 8 * kk;
       const uint16_t* vr = v_cache + ((page * G + g) * dv + li) * kPageB + 4 * kk;
 #pragma unroll
@@ -304,6 +317,8 @@ __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
           acc[i][c] = T::mfma(make_uint4(pw[i][0], pw[i][1], pw[i][2], pw[i][3]), v4, acc[i][c]);
       }
     }
+    pg[0] = npg[0];
+    pg[1] = npg[1];
   }
   // C layout: this lane holds rows 4 kk + r of column li of every 16-column block
 #pragma unroll

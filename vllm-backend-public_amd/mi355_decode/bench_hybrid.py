@@ -487,7 +487,7 @@ def tafisun_kernel_table(width: int, prompt_len: int, batch: int) -> list:
             b_t = bt
         rep = H // G
         hb = 4 if rep % 4 == 0 else 3 if rep % 3 == 0 else 2 if rep % 2 == 0 else 1
-        nsb = max(min(16, block // 64, 2048 // max(int(tiles.shape[0]) * G * (rep // hb), 1)), 1)
+        nsb = max(min(16, block // 64, 1024 // max(int(tiles.shape[0]) * G * (rep // hb), 1)), 1)
         nsw = max(min(16, 2048 // max(int(tiles.shape[0]) * G * max(rep // 4, 1), 1)), 1)
         part = torch.empty(nsw * T * H * d, device=dev)
         o = torch.empty(T, H * d, device=dev, dtype=bf)

@@ -446,7 +446,10 @@ class HybridRunner(ModelRunner):
         hb = 4 if rep % 4 == 0 else 3 if rep % 3 == 0 else 2 if rep % 2 == 0 else 1
         waves = int(b.tiles.shape[0]) * a.kv_heads * (rep // hb)
         span = a.block if a.block > 0 else self.max_model_len
-        n = min(self.MAX_KEY_SPLITS, max(span // 64, 1), max(2048 // max(waves, 1), 1))
+        # about a wave per SIMD: every further split costs its fp32 partial sums and their merge (measured: a
+        # 2048-token prompt of 16 heads 203 / 117 / 130 / 161 us with 1 / 2 / 4 / 8 splits, 32 decoded rows
+        # 148 / 83 / 51 / 36 / 43 us with 1 / 2 / 4 / 8 / 16)
+        n = min(self.MAX_KEY_SPLITS, max(span // 64, 1), max(1024 // max(waves, 1), 1))
         return n if n > 1 else 0
 
     def kv_cache_bytes_per_block(self) -> int:

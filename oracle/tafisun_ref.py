@@ -11,9 +11,9 @@ Notation.  W: model width; rms(x; g) = x / sqrt(mean(x^2) + eps) * g.
     logits = head rms(x; final.norm)
 
 Mixers
-  * "attention": grouped-query softmax attention whose values ARE the keys as projected (no value
-    projection); queries and keys get a per-head RMS norm with one weight vector shared by the
-    heads; no rotation; score_ij = q_i.k_j * scale - r1_h ln(1 + r2_h (i - j)); position i sees
+  * "attention": grouped-query softmax attention with no value projection (the key projection, taken
+    ahead of its norm, doubles as the value); queries and keys get a per-head RMS norm with one weight
+    vector shared by the heads; no rotation; score_ij = q_i.k_j * scale - r1_h ln(1 + r2_h (i - j)); position i sees
     j <= i of its own block of `size` positions (blocks counted from position 0); the concatenated
     heads are multiplied by sigmoid(G h) before the output projection.
   * "mingru": z = sigmoid(Z h + bz), u = X h + bx, c = u + 1/2 (u >= 0) or sigmoid(u) (u < 0);
@@ -72,7 +72,7 @@ def block_attention(q, k, wq, wk, r1, r2, scale, size, eps, gate=None):
     """q [T, H, d], k [T, G, d] as projected.  Returns the gated, concatenated heads [T, H * d]."""
     T, H, d = q.shape
     G = k.shape[1]
-    v = k                                                   # the values are the keys before their norm
+    v = k                                                   # the un-normed key projection doubles as the value
     qn, kn = rms_norm(q, wq, eps), rms_norm(k, wk, eps)
     rep = H // G
     ke, ve = kn.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)

@@ -146,8 +146,8 @@ class BlockAttnSpec:
     """Softmax attention inside blocks of `block` positions (position i sees j <= i with
     i // block == j // block; block 0: plain causal), grouped heads, no rotation: the score is
     q.k * scale - r1[h] * ln(1 + r2[h] * (i - j)).  Queries and keys get an RMS norm per head with one
-    weight vector shared by the heads.  values_are_keys: there is no value projection, the values
-    are the keys as projected, before their norm (then vdim == dim).  The concatenated heads are
+    weight vector shared by the heads.  values_are_keys: no value projection exists; the key
+    projection, taken ahead of its norm, doubles as the value (then vdim == dim).  The concatenated heads are
     multiplied by a sigmoid gate of their own width."""
     heads: int
     kv_heads: int

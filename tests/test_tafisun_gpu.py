@@ -57,6 +57,13 @@ CONFIGS = {
              "layers": [{"type": "attention", "mixer": _attn(8, 2, 64, 48, 0.125), "mlp": _moe(8, 2, 2, 5, 2, 256, 2.0, 1.5, shared=(128, 1.5))},
                         {"type": "mingru", "mixer": {"width": 512}, "mlp": {"kind": "dense", "ff": 1024}},
                         {"type": "attention", "mixer": _attn(6, 2, 32, 33, 0.2), "mlp": _moe(16, 0, 4, 4, 1, 128, 4.0)}]},
+    # a width that is no multiple of 8, head and expert sizes that no matrix-core tile covers, five ungrouped heads,
+    # an eight-channel recurrence, seven experts of which three run
+    "odd": {"architecture": "Tafisun", "width": 90, "vocab": 101, "norm": {"eps": 1e-5}, "embedding": _bigram(97, 11, 3),
+            "layers": [{"type": "mingru", "mixer": {"width": 77}, "mlp": _moe(5, 1, 2, 2, 1, 30, 1.5, 1.2, shared=(22, 1.0))},
+                       {"type": "attention", "mixer": _attn(5, 5, 24, 96), "mlp": {"kind": "dense", "ff": 50}},
+                       {"type": "attention", "mixer": _attn(4, 2, 48, 10), "mlp": _moe(7, 0, 3, 1, 1, 18, 2.0)},
+                       {"type": "mingru", "mixer": {"width": 8}, "mlp": None}]},
 }
 _cache = {}
 

@@ -629,3 +629,49 @@ def test_served_from_a_model_directory(tmp_path):
             proc.wait(timeout=20)
         except subprocess.TimeoutExpired:
             os.killpg(proc.pid, signal.SIGKILL)
+
+
+def test_trace_replay_program(tmp_path):
+    """bin/trace_run on a model directory of this design: steps as JSON lines on standard input (a
+    portion beside a single token, a request that ends and one that takes its place), float32 logits
+    of the wanted rows per step on disk, a 'done <step>' line after every step."""
+    import json
+    import os
+    import subprocess
+    from safetensors.torch import save_file
+    from conftest import ROOT
+    name = "plain"
+    cfg, w = CONFIGS[name], _weights(name)
+    model_dir, out_dir = tmp_path / "model", tmp_path / "out"
+    model_dir.mkdir()
+    json.dump(cfg, open(model_dir / "config.json", "w"))
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in w.items()}, str(model_dir / "model.safetensors"))
+    a, b, c = _tokens(name, 50, 1), _tokens(name, 20, 2), _tokens(name, 9, 3)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:33], "want": [0, 32]}, {"id": "b", "tokens": b[:1], "want": [0]}], "end": []},
+             {"step": 1, "entries": [{"id": "b", "tokens": b[1:], "want": [18]}, {"id": "a", "tokens": a[33:34], "want": [0]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[34:36], "want": []}], "end": []},
+             {"step": 3, "entries": [{"id": "c", "tokens": c, "want": [8]}, {"id": "a", "tokens": a[36:], "want": [13]}], "end": ["a", "c"]}]
+    p = subprocess.Popen([os.path.join(ROOT, "bin", "trace_run"), "--model", str(model_dir), "--dtype", "float32", "--out", str(out_dir),
+                          "--max-tokens", "128"], stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    try:
+        for st in steps:
+            p.stdin.write(json.dumps(st) + "\n")
+            p.stdin.flush()
+            while True:
+                line = p.stdout.readline()
+                assert line, "the program ended early"
+                if line.strip() == f"done {st['step']}":
+                    break
+        p.stdin.close()
+        assert p.wait(timeout=60) == 0
+    finally:
+        if p.poll() is None:
+            p.kill()
+    V = cfg["vocab"]
+    ra, rb, rc = _ref(name, a), _ref(name, b), _ref(name, c)
+    want = {0: [ra[0], ra[32], rb[0]], 1: [rb[19], ra[33]], 3: [rc[8], ra[49]]}
+    assert not (out_dir / "2.f32").exists()
+    for n, rows in want.items():
+        got = np.fromfile(out_dir / f"{n}.f32", dtype="<f4").reshape(-1, V)
+        assert got.shape[0] == len(rows)
+        _close(got, np.stack(rows))

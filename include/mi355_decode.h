@@ -740,6 +740,8 @@ int32_t mi355_allreduce_oneshot_destroy(void* comm);
  * keeps the residual in the model's 16-bit type).  `dtype` is the storage type of activations and
  * weights: MI355_BF16, MI355_F16 or MI355_F32; sums, means and transcendentals are fp32 always.
  *   embed_scale_f32       resid[t] = embed[ids[t]] * scale
+ *   embed_scale_pos_f32   resid[t] = embed[ids[t]] * scale + pos_table[positions[t]] (learned positions,
+ *                         [max_pos, width] in `dtype`)
  *   resid_add_f32         resid[t] += other[t] (fp32) + rows[t] (dtype) + vec (one row, dtype); each may be null
  *   add_rms_norm_f32      resid += add (may be null); out = resid / sqrt(mean(resid^2) + eps) * w,
  *                         w one number (weight_numel 1) or one per column (weight_numel == width)
@@ -752,6 +754,9 @@ int32_t mi355_allreduce_oneshot_destroy(void* comm);
  */
 int32_t mi355_embed_scale_f32(float* out, const void* embed, const int64_t* ids, int64_t num_tokens,
                               int32_t width, int64_t vocab, float scale, int32_t dtype, void* stream);
+int32_t mi355_embed_scale_pos_f32(float* out, const void* embed, const void* pos_table, const int64_t* ids,
+                                  const int64_t* positions, int64_t num_tokens, int32_t width,
+                                  int64_t vocab, int64_t max_pos, float scale, int32_t dtype, void* stream);
 int32_t mi355_resid_add_f32(float* resid, const float* other, const void* rows, const void* vec,
                             int64_t num_tokens, int32_t width, int32_t dtype, void* stream);
 int32_t mi355_add_rms_norm_f32(void* out, float* resid, const void* add, const void* weight,
@@ -777,7 +782,8 @@ int32_t mi355_softcap(void* z, int64_t numel, float cap, int32_t dtype, void* st
  *   rope_partial_kv_write  rotates the first rot_dims coordinates of every q and k head (coordinate
  *                          i with i + rot_dims / 2) by the fp32 table cos_sin [max_pos, rot_dims]
  *                          (cos | sin), q in place, k into its page; v is copied into its page;
- *                          rows with slot < 0 store nothing
+ *                          rows with slot < 0 store nothing.  k, v and both caches null: queries only
+ *                          (a layer that attends to another layer's pages)
  *   sigmoid_window_attn    out[t, h] = sigmoid(gate[t, h]) * sum over keys j of the row's sequence with
  *                          0 <= p - j < window of sigmoid(q.k_j * scale * temp[h] + bias[h]) * v_j
  *                          (gate may be null); weights are not normalised over keys.  With `tiles`
@@ -951,7 +957,9 @@ int32_t mi355_latent_window_attn(void* out, int64_t out_stride, int64_t out_head
  *                     of the `keep` best of `groups` groups of neighbouring experts (a group scores
  *                     the sum of its two largest score + correction, or with `group_max` the
  *                     largest); ids [tokens, top], weights [tokens, top] = the chosen experts'
- *                     scores times weight_scale (no correction, not renormalised)
+ *                     scores times weight_scale (no correction, not renormalised).  softmax 2: the
+ *                     score is the logit itself and the weights are a softmax over the chosen logits
+ *                     alone, times weight_scale
  *   moe_sort          routed rows by expert: offsets [experts + 1], perm[position] = row,
  *                     inv[row] = position
  *   moe_gather_rows   xs[position] = x[perm[position] / top] for num_rows positions (pad_to 0); with
@@ -962,6 +970,8 @@ int32_t mi355_latent_window_attn(void* out, int64_t out_stride, int64_t out_head
  *                     limit): g * sigmoid(1.702 g) * (u + 1) (act 1)
  *   moe_down_rows     y[position] = Wd[e] act[position]; w_down [experts, width, ff]
  *   moe_silu_and_mul  out = a(x[:, :ff], x[:, ff:])
+ *   gated_act_rows    out[r, :ff] = a(gate[r, :ff], up[r, :ff]): gate and up rows in_stride apart, out
+ *                     rows out_stride apart (column slices of wider buffers)
  *   moe_combine       out[t] = sum_k weights[t, k] * y[inv[t * top + k]]; with pad_to > 0, y holds every
  *                     expert's rows padded to pad_to (ids and offsets locate them).  x not null: a
  *                     chosen id >= num_real is an identity expert, its row is x[t].  shared not null:
@@ -983,6 +993,9 @@ int32_t mi355_moe_down_rows(void* y, const void* act, const void* w_down, const 
                             int32_t experts, int32_t width, int32_t ff, int32_t dtype, void* stream);
 int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_rows, int32_t ff, int32_t act_fn,
                                float limit, int32_t dtype, void* stream);
+int32_t mi355_gated_act_rows(void* out, int64_t out_stride, const void* gate, const void* up,
+                             int64_t in_stride, int64_t num_rows, int32_t ff, int32_t act_fn, float limit,
+                             int32_t dtype, void* stream);
 int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const float* weights,
                           const int32_t* ids, const int32_t* offsets, int32_t pad_to,
                           int64_t num_tokens, int32_t top, int32_t width, const void* x,
@@ -1003,7 +1016,9 @@ int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const fl
  *   softmax_bias_attn     out[t,h] = sigmoid(gate) * sum_j softmax_j(q.k_j * scale - r1[h] ln(1 + r2[h]
  *                         (p - j))) v_j over the keys j <= p with j >= (p / block) * block (block 0: all)
  *                         and, window > 0, j > p - window.  gate: one number per head or
- *                         (gate_per_channel) per output channel; r1 / r2 null: no penalty.  tiles as for
+ *                         (gate_per_channel) per output channel; r1 / r2 null: no penalty.  sink (fp32
+ *                         [heads], may be null): one more term exp(sink[h]) in the softmax denominator,
+ *                         without a value.  Output rows are out_stride elements apart.  tiles as for
  *                         sigmoid_window_attn; workspace (softmax_bias_attn_workspace floats) with
  *                         num_splits > 1 spreads a tile's keys over that many workgroups
  *   mingru_scan           S <- (1 - z) S + z c per channel, z = sigmoid(zp + z_bias), u = xp + x_bias,
@@ -1037,7 +1052,8 @@ int32_t mi355_softmax_bias_attn(void* out, const void* q, int64_t q_stride, cons
                                 int32_t gate_per_channel, int64_t num_tokens, int32_t num_heads,
                                 int32_t num_kv_heads, int32_t head_dim, int32_t v_dim, int32_t block,
                                 int32_t window, float scale, const int32_t* tiles, int32_t num_tiles,
-                                float* workspace, int32_t num_splits, int32_t dtype, void* stream);
+                                float* workspace, int32_t num_splits, const float* sink,
+                                int64_t out_stride, int32_t dtype, void* stream);
 int32_t mi355_mingru_scan(void* out, const void* proj, int64_t stride, int32_t z_off, int32_t x_off,
                           int32_t g_off, const float* z_bias, const float* x_bias, float* state,
                           const int32_t* cu_seqlens, const int64_t* positions,

@@ -9,6 +9,9 @@
 //                         over the keys j <= p of p's block: lo = (p / block) * block (block 0: lo = 0), and
 //                         with a window also j > p - window.  Blocks are counted from position 0 of the
 //                         sequence.  gate: sigmoid of one number per head or per output channel.
+//                         sink (fp32, one score per head, may be null): the softmax denominator holds one
+//                         more term exp(sink[h]) that carries no value.  Output rows are out_stride apart
+//                         (a column slice of a wider buffer is fine).
 // Norms, scores, penalties, softmax and accumulators are fp32; pages and activations are stored in
 // the dtype argument's type.  K pages [blocks, kv_heads, 16, dim], V pages [blocks, kv_heads, vdim, 16].
 #include "common.h"
@@ -74,7 +77,7 @@ __global__ __launch_bounds__(64) void softmax_bias_attn_kernel(
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ tok_seq,
     const int64_t* __restrict__ positions, const float* __restrict__ r1, const float* __restrict__ r2,
     const typename Elem<T>::S* __restrict__ gate, int64_t gate_stride, int gate_per_channel, int H, int G, int d, int dv,
-    int block, int window, float scale) {
+    int block, int window, float scale, const float* __restrict__ sink, int64_t out_stride) {
   extern __shared__ float lds[];                        // q [d] | w [64]
   float* qs = lds;
   float* ws = lds + d;
@@ -129,6 +132,14 @@ __global__ __launch_bounds__(64) void softmax_bias_attn_kernel(
     }
     __syncthreads();
   }
+  if (sink != nullptr) {                                // one more term in the denominator, no value
+    const float sk = MI355_LD(float, sink, sink + h);
+    const float mn = fmaxf(m, sk);
+    const float corr = expf(m - mn);
+    l = l * corr + expf(sk - mn);
+#pragma unroll
+    for (int i = 0; i < DV_PER_LANE; ++i) acc[i] *= corr;
+  }
   const float inv = 1.0f / l;
 #pragma unroll
   for (int i = 0; i < DV_PER_LANE; ++i) {
@@ -137,7 +148,7 @@ __global__ __launch_bounds__(64) void softmax_bias_attn_kernel(
     float gt = 1.0f;
     if (gate != nullptr)
       gt = 1.0f / (1.0f + expf(-MI355_LDF(T, gate, gate + t * gate_stride + (gate_per_channel ? h * dv + c : h))));
-    MI355_STF(T, out, out + (t * H + h) * dv + c, acc[i] * inv * gt);
+    MI355_STF(T, out, out + t * out_stride + static_cast<int64_t>(h) * dv + c, acc[i] * inv * gt);
   }
 }
 
@@ -158,7 +169,7 @@ __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
     const int32_t* __restrict__ tiles, int num_tiles, const int64_t* __restrict__ positions, const float* __restrict__ r1,
     const float* __restrict__ r2, const uint16_t* __restrict__ gate, int64_t gate_stride, int gate_per_channel, int H, int G,
     int d, int dv, int block, int window, float scale, float* __restrict__ part_acc, float* __restrict__ part_ml,
-    int64_t total_rows) {
+    int64_t total_rows, const float* __restrict__ sink, int64_t out_stride) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int tile = blockIdx.x * (blockDim.x >> 6) + wave;
   if (tile >= num_tiles) return;                        // (no workgroup barrier below)
@@ -344,7 +355,15 @@ __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
       }
       continue;
     }
-    const float f = 1.0f / lt;
+    float f = 1.0f / lt;
+    if (sink != nullptr) {
+      // the extra term of the denominator, base 2 like the maxima: numerator and denominator are both
+      // relative to m[i], so the accumulators only need the ratio
+      const float sk = MI355_LD(float, sink, sink + h) * kLog2eB;
+      const float mn = fmaxf(m[i], sk);
+      const float cm = __builtin_amdgcn_exp2f(m[i] - mn);
+      f = cm / (lt * cm + __builtin_amdgcn_exp2f(sk - mn));
+    }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int rr = 4 * kk + r;
@@ -358,7 +377,8 @@ __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
         if (c >= cbs) continue;
         float gt = gh;
         if (gate != nullptr && gate_per_channel) gt = 1.0f / (1.0f + expf(-T::to_f(MI355_LD(uint16_t, gate, gr + 16 * c + li))));
-        MI355_ST(uint16_t, out, out + ((row0 + rr) * H + h) * dv + 16 * c + li, T::from_f(acc[i][c][r] * fr * gt));
+        MI355_ST(uint16_t, out, out + (row0 + rr) * out_stride + static_cast<int64_t>(h) * dv + 16 * c + li,
+                 T::from_f(acc[i][c][r] * fr * gt));
       }
     }
   }
@@ -369,7 +389,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void bias_attn_merge_kernel(uint16_t* __restrict__ out, const float* __restrict__ part_acc,
                                                               const float* __restrict__ part_ml,
                                                               const uint16_t* __restrict__ gate, int64_t gate_stride,
-                                                              int gate_per_channel, int64_t rows, int H, int dv, int splits) {
+                                                              int gate_per_channel, int64_t rows, int H, int dv, int splits,
+                                                              const float* __restrict__ sink, int64_t out_stride) {
   const int64_t pairs = rows * H, total = pairs * dv;
   for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
        i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
@@ -386,10 +407,17 @@ __global__ __launch_bounds__(256) void bias_attn_merge_kernel(uint16_t* __restri
       den += MI355_LD(float, part_ml, ml + 1) * e;
       num += MI355_LD(float, part_acc, part_acc + (z * pairs + pair) * dv + c) * e;
     }
+    if (sink != nullptr) {
+      const float sk = MI355_LD(float, sink, sink + h) * kLog2eB;
+      const float mn = fmaxf(M, sk);
+      const float cm = __builtin_amdgcn_exp2f(M - mn);
+      num *= cm;
+      den = den * cm + __builtin_amdgcn_exp2f(sk - mn);
+    }
     float v = num / den;
     if (gate != nullptr)
       v /= 1.0f + expf(-T::to_f(MI355_LD(uint16_t, gate, gate + row * gate_stride + (gate_per_channel ? h * dv + c : h))));
-    MI355_ST(uint16_t, out, out + i, T::from_f(v));
+    MI355_ST(uint16_t, out, out + row * out_stride + static_cast<int64_t>(h) * dv + c, T::from_f(v));
   }
 }
 
@@ -430,7 +458,7 @@ static void launch_bias_attn(hipStream_t s, void* out, const void* q, int64_t q_
                              const void* v_cache, const int32_t* block_tables, int32_t max_blocks, const int32_t* tok_seq,
                              const int64_t* positions, const float* r1, const float* r2, const void* gate,
                              int64_t gate_stride, int gate_per_channel, int64_t T, int H, int G, int d, int dv, int block,
-                             int window, float scale) {
+                             int window, float scale, const float* sink, int64_t out_stride) {
   typedef typename Elem<TT>::S E;
   const dim3 grid(static_cast<unsigned>(T), static_cast<unsigned>(H));
   const size_t lds = (static_cast<size_t>(d) + 64) * sizeof(float);
@@ -438,7 +466,8 @@ static void launch_bias_attn(hipStream_t s, void* out, const void* q, int64_t q_
   hipLaunchKernelGGL((softmax_bias_attn_kernel<TT, N>), grid, dim3(64), lds, s, static_cast<E*>(out),              \
                      static_cast<const E*>(q), q_stride, static_cast<const E*>(k_cache),                           \
                      static_cast<const E*>(v_cache), block_tables, max_blocks, tok_seq, positions, r1, r2,         \
-                     static_cast<const E*>(gate), gate_stride, gate_per_channel, H, G, d, dv, block, window, scale)
+                     static_cast<const E*>(gate), gate_stride, gate_per_channel, H, G, d, dv, block, window, scale, \
+                     sink, out_stride)
   if (dv <= 64) MI355_BATTN(1);
   else if (dv <= 128) MI355_BATTN(2);
   else MI355_BATTN(4);
@@ -456,7 +485,8 @@ extern "C" int32_t mi355_softmax_bias_attn(void* out, const void* q, int64_t q_s
                                            int32_t gate_per_channel, int64_t num_tokens, int32_t num_heads,
                                            int32_t num_kv_heads, int32_t head_dim, int32_t v_dim, int32_t block,
                                            int32_t window, float scale, const int32_t* tiles, int32_t num_tiles,
-                                           float* workspace, int32_t num_splits, int32_t dtype, void* stream) {
+                                           float* workspace, int32_t num_splits, const float* sink, int64_t out_stride,
+                                           int32_t dtype, void* stream) {
   MI355_REQUIRE(out && q && k_cache && v_cache && block_tables && tok_seq && positions, MI355_ERR_INVALID,
                 "softmax_bias_attn: null pointer");
   MI355_REQUIRE((r1 == nullptr) == (r2 == nullptr), MI355_ERR_INVALID, "softmax_bias_attn: r1 and r2 go together");
@@ -467,6 +497,8 @@ extern "C" int32_t mi355_softmax_bias_attn(void* out, const void* q, int64_t q_s
                 "softmax_bias_attn: v_dim %d (at most 256), head_dim %d", v_dim, head_dim);
   MI355_REQUIRE(gate == nullptr || gate_stride >= (gate_per_channel ? static_cast<int64_t>(num_heads) * v_dim : num_heads),
                 MI355_ERR_INVALID, "softmax_bias_attn: gate rows shorter than the gate");
+  MI355_REQUIRE(out_stride >= static_cast<int64_t>(num_heads) * v_dim, MI355_ERR_INVALID,
+                "softmax_bias_attn: output rows shorter than heads * v_dim");
   REQ_DTYPE(dtype);
   if (num_tokens == 0) return MI355_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -489,7 +521,7 @@ extern "C" int32_t mi355_softmax_bias_attn(void* out, const void* q, int64_t q_s
                      static_cast<const uint16_t*>(k_cache), static_cast<const uint16_t*>(v_cache), block_tables,    \
                      max_blocks, tiles, num_tiles, positions, r1, r2, static_cast<const uint16_t*>(gate),           \
                      gate_stride, gate_per_channel, num_heads, num_kv_heads, head_dim, v_dim, block, window, scale, \
-                     part_acc, part_ml, num_tokens)
+                     part_acc, part_ml, num_tokens, sink, out_stride)
 #define MI355_BMFMA_HB(TT)                                                                                          \
   do {                                                                                                              \
     if (hb == 4) MI355_BMFMA(TT, 4);                                                                                \
@@ -502,7 +534,7 @@ extern "C" int32_t mi355_softmax_bias_attn(void* out, const void* q, int64_t q_s
                          dim3(static_cast<unsigned>((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256)),      \
                          dim3(256), 0, s, static_cast<uint16_t*>(out), part_acc, part_ml,                           \
                          static_cast<const uint16_t*>(gate), gate_stride, gate_per_channel, num_tokens, num_heads,  \
-                         v_dim, num_splits);                                                                        \
+                         v_dim, num_splits, sink, out_stride);                                                      \
     }                                                                                                               \
   } while (0)
     if (dtype == MI355_BF16) MI355_BMFMA_HB(BF16); else MI355_BMFMA_HB(F16);
@@ -513,6 +545,6 @@ extern "C" int32_t mi355_softmax_bias_attn(void* out, const void* q, int64_t q_s
   MI355_DISPATCH_DTYPE3(dtype, launch_bias_attn<TT>(s, out, q, q_stride, k_cache, v_cache, block_tables, max_blocks,
                                                    tok_seq, positions, r1, r2, gate, gate_stride, gate_per_channel,
                                                    num_tokens, num_heads, num_kv_heads, head_dim, v_dim, block, window,
-                                                   scale));
+                                                   scale, sink, out_stride));
   return check_launch("softmax_bias_attn");
 }

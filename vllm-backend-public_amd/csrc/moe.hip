@@ -1,6 +1,7 @@
 // Mixture-of-experts feed-forward: routing, the expert-sorted row order, and the expert products for
 // steps of few rows.
-//   moe_route           scores from fp32 router logits (a sigmoid each, or a softmax over all of them);
+//   moe_route           scores from fp32 router logits (a sigmoid each, a softmax over all of them, or the
+//                       logits themselves with a softmax over the chosen ones as weights);
 //                       experts are picked by score + correction among the experts of the best `keep` of
 //                       `count` groups of neighbours (a group scores the sum of its two best, or its
 //                       best), and weighted by the score without correction, times a constant
@@ -26,6 +27,16 @@ namespace mi355 {
 constexpr int kMaxGroups = 64;
 constexpr int kMaxTop = 16;
 
+// softmax == 2: the stored weights are the chosen logits; they become a softmax over the chosen
+// alone, times wscale.  The thread that stored them rewrites them.
+__device__ __forceinline__ void chosen_softmax(float* w, [[maybe_unused]] const float* base, int top, float wscale) {
+  float mx = -__builtin_inff();
+  for (int r = 0; r < top; ++r) mx = fmaxf(mx, MI355_LD(float, base, w + r));
+  float sum = 0.f;
+  for (int r = 0; r < top; ++r) sum += expf(MI355_LD(float, base, w + r) - mx);
+  for (int r = 0; r < top; ++r) MI355_ST(float, base, w + r, expf(MI355_LD(float, base, w + r) - mx) / sum * wscale);
+}
+
 __global__ __launch_bounds__(64) void moe_route_kernel(int32_t* __restrict__ ids, float* __restrict__ wts,
                                                        const float* __restrict__ z, int64_t z_stride,
                                                        const float* __restrict__ corr, int64_t T, int E, int top, int count,
@@ -36,14 +47,14 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int32_t* __restrict__ ids
   const int per = E / count;
   const float ninf = -__builtin_inff();
   float zmax = ninf, zsum = 1.0f;
-  if (softmax) {
+  if (softmax == 1) {
     for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, MI355_LD(float, z, zr + e));
     zsum = 0.f;
     for (int e = 0; e < E; ++e) zsum += expf(MI355_LD(float, z, zr + e) - zmax);
   }
   auto score = [&](int e) {
     const float v = MI355_LD(float, z, zr + e);
-    return softmax ? expf(v - zmax) / zsum : 1.0f / (1.0f + expf(-v));
+    return softmax == 2 ? v : softmax ? expf(v - zmax) / zsum : 1.0f / (1.0f + expf(-v));
   };
   auto choice = [&](int e) { return score(e) + MI355_LD(float, corr, corr + e); };
   // the groups that stay: `keep` rounds of picking the best group not yet picked
@@ -81,8 +92,9 @@ __global__ __launch_bounds__(64) void moe_route_kernel(int32_t* __restrict__ ids
     }
     picked[r] = best;
     MI355_ST(int32_t, ids, ids + t * top + r, best);
-    MI355_ST(float, wts, wts + t * top + r, score(best) * wscale);
+    MI355_ST(float, wts, wts + t * top + r, score(best) * (softmax == 2 ? 1.0f : wscale));
   }
+  if (softmax == 2) chosen_softmax(wts + t * top, wts, top, wscale);
 }
 
 // (value, index) maximum over the wave, every lane gets it; ties go to the lower index
@@ -111,7 +123,7 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(int32_t* __restrict
   const float ninf = -__builtin_inff();
   const int per = E / count;
   float zmax = ninf, zsum = 1.0f;
-  if (softmax) {                                        // over all router outputs, in fp32
+  if (softmax == 1) {                                   // over all router outputs, in fp32
 #pragma unroll
     for (int i = 0; i < EPL; ++i)
       if (lane + 64 * i < E) zmax = fmaxf(zmax, MI355_LD(float, z, zr + lane + 64 * i));
@@ -125,7 +137,7 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(int32_t* __restrict
   }
   auto score = [&](int e) {
     const float v = MI355_LD(float, z, zr + e);
-    return softmax ? expf(v - zmax) / zsum : 1.0f / (1.0f + expf(-v));
+    return softmax == 2 ? v : softmax ? expf(v - zmax) / zsum : 1.0f / (1.0f + expf(-v));
   };
   float c[EPL];
 #pragma unroll
@@ -175,9 +187,10 @@ __global__ __launch_bounds__(256) void moe_route_wave_kernel(int32_t* __restrict
       if (lane + 64 * i == e) c[i] = ninf;              // taken
     if (live && lane == 0) {
       MI355_ST(int32_t, ids, ids + t * top + r, e);
-      MI355_ST(float, wts, wts + t * top + r, score(e) * wscale);
+      MI355_ST(float, wts, wts + t * top + r, score(e) * (softmax == 2 ? 1.0f : wscale));
     }
   }
+  if (softmax == 2 && live && lane == 0) chosen_softmax(wts + t * top, wts, top, wscale);
 }
 
 // one workgroup: counts, an exclusive prefix, then a position for every row
@@ -421,6 +434,23 @@ __global__ __launch_bounds__(256) void moe_silu_and_mul_kernel(typename Elem<T>:
   }
 }
 
+// the same activation for rows whose gate and up parts are column slices of a wider buffer, into a
+// column slice of another
+template <typename T>
+__global__ __launch_bounds__(256) void gated_act_rows_kernel(typename Elem<T>::S* __restrict__ out, int64_t out_stride,
+                                                             const typename Elem<T>::S* __restrict__ gate,
+                                                             const typename Elem<T>::S* __restrict__ up, int64_t in_stride,
+                                                             int64_t rows, int F, int act, float limit) {
+  const int64_t total = rows * F;
+  for (int64_t i = blockIdx.x * static_cast<int64_t>(blockDim.x) + threadIdx.x; i < total;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t r = i / F;
+    const int f = static_cast<int>(i % F);
+    MI355_STF(T, out, out + r * out_stride + f,
+              gated_act(MI355_LDF(T, gate, gate + r * in_stride + f), MI355_LDF(T, up, up + r * in_stride + f), act, limit));
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_kernel(typename Elem<T>::S* __restrict__ out,
                                                           const typename Elem<T>::S* __restrict__ y,
@@ -591,6 +621,22 @@ extern "C" int32_t mi355_moe_silu_and_mul(void* out, const void* x, int64_t num_
                                                   static_cast<Elem<TT>::S*>(out), static_cast<const Elem<TT>::S*>(x),
                                                   num_rows, ff, act, limit));
   return check_launch("moe_silu_and_mul");
+}
+
+extern "C" int32_t mi355_gated_act_rows(void* out, int64_t out_stride, const void* gate, const void* up, int64_t in_stride,
+                                        int64_t num_rows, int32_t ff, int32_t act, float limit, int32_t dtype, void* stream) {
+  MI355_REQUIRE(out && gate && up, MI355_ERR_INVALID, "gated_act_rows: null pointer");
+  MI355_REQUIRE(num_rows >= 0 && ff > 0 && out_stride >= ff && in_stride >= ff, MI355_ERR_INVALID, "gated_act_rows: sizes");
+  REQ_DTYPE(dtype);
+  if (num_rows == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t blocks = (num_rows * ff + 255) / 256;
+  const dim3 grid(static_cast<unsigned>(blocks > 65536 ? 65536 : blocks));
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((gated_act_rows_kernel<TT>), grid, dim3(256), 0, s,
+                                                  static_cast<Elem<TT>::S*>(out), out_stride,
+                                                  static_cast<const Elem<TT>::S*>(gate), static_cast<const Elem<TT>::S*>(up),
+                                                  in_stride, num_rows, ff, act, limit));
+  return check_launch("gated_act_rows");
 }
 
 extern "C" int32_t mi355_moe_combine(void* out, const void* y, const int32_t* inv, const float* weights, const int32_t* ids,

@@ -1,5 +1,6 @@
 // Pointwise and normalisation kernels for decoders that keep the residual stream in fp32:
 //   embed_scale_f32          resid = embed[id] * scale
+//   embed_scale_pos_f32      resid = embed[id] * scale + pos_table[position]      (learned positions)
 //   resid_add_f32            resid += other (fp32 rows) + rows (activation rows) + vec (one row, broadcast)
 //   add_rms_norm_f32         resid += add; out = resid / rms(resid) * w      (w: one number or a vector)
 //   rms_norm_mix_f32         resid += alpha * (xa / rms(xa) * wa + xb / rms(xb) * wb)
@@ -26,6 +27,22 @@ __global__ __launch_bounds__(256) void embed_scale_f32_kernel(float* __restrict_
   const int64_t id = MI355_LD(int64_t, ids, ids + t);
   for (int c = threadIdx.x; c < W; c += blockDim.x)
     MI355_ST(float, out, out + t * W + c, MI355_LDF(T, embed, embed + id * W + c) * scale);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void embed_scale_pos_f32_kernel(float* __restrict__ out,
+                                                                  const typename Elem<T>::S* __restrict__ embed,
+                                                                  const typename Elem<T>::S* __restrict__ pos_table,
+                                                                  const int64_t* __restrict__ ids,
+                                                                  const int64_t* __restrict__ positions, int W,
+                                                                  int64_t max_pos, float scale) {
+  const int64_t t = blockIdx.x;
+  const int64_t id = MI355_LD(int64_t, ids, ids + t);
+  int64_t p = MI355_LD(int64_t, positions, positions + t);
+  p = p < 0 ? 0 : (p >= max_pos ? max_pos - 1 : p);     // (padding rows of a captured step: any row will do)
+  for (int c = threadIdx.x; c < W; c += blockDim.x)
+    MI355_ST(float, out, out + t * W + c,
+             MI355_LDF(T, embed, embed + id * W + c) * scale + MI355_LDF(T, pos_table, pos_table + p * W + c));
 }
 
 template <typename T>
@@ -361,6 +378,21 @@ extern "C" int32_t mi355_embed_scale_f32(float* out, const void* embed, const in
   MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((embed_scale_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s, out,
                                                   static_cast<const Elem<TT>::S*>(embed), ids, width, scale));
   return check_launch("embed_scale_f32");
+}
+
+extern "C" int32_t mi355_embed_scale_pos_f32(float* out, const void* embed, const void* pos_table, const int64_t* ids,
+                                             const int64_t* positions, int64_t num_tokens, int32_t width, int64_t vocab,
+                                             int64_t max_pos, float scale, int32_t dtype, void* stream) {
+  MI355_REQUIRE(out && embed && pos_table && ids && positions, MI355_ERR_INVALID, "embed_scale_pos_f32: null pointer");
+  MI355_REQUIRE(num_tokens >= 0 && width > 0 && vocab > 0 && max_pos > 0, MI355_ERR_INVALID, "embed_scale_pos_f32: sizes");
+  REQ_DTYPE(dtype);
+  if (num_tokens == 0) return MI355_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  MI355_DISPATCH_DTYPE3(dtype, hipLaunchKernelGGL((embed_scale_pos_f32_kernel<TT>), dim3(num_tokens), dim3(256), 0, s, out,
+                                                  static_cast<const Elem<TT>::S*>(embed),
+                                                  static_cast<const Elem<TT>::S*>(pos_table), ids, positions, width,
+                                                  max_pos, scale));
+  return check_launch("embed_scale_pos_f32");
 }
 
 extern "C" int32_t mi355_embed_bigram_pos_f32(float* out, const void* embed, const void* bigram, const int64_t* ids,

@@ -47,7 +47,7 @@ __global__ __launch_bounds__(256) void rope_partial_kv_write_kernel(
     MI355_STF(T, q, row + j, a * c - b * s);
     MI355_STF(T, q, row + half + j, b * c + a * s);
   }
-  if (slot < 0) return;
+  if (slot < 0 || k == nullptr) return;                 // k null: a layer that reads another layer's pages
   const int64_t page = slot / kPage, off = slot % kPage;
   for (int i = threadIdx.x; i < G * d; i += blockDim.x) {
     const int g = i / d, j = i % d;
@@ -937,15 +937,16 @@ extern "C" int32_t mi355_rope_partial_kv_write(void* q, int64_t q_stride, const 
                                                void* v_cache, int64_t num_tokens, int32_t num_heads,
                                                int32_t num_kv_heads, int32_t head_dim, int32_t v_dim, int32_t rot_dims,
                                                int32_t dtype, void* stream) {
-  MI355_REQUIRE(q && k && v && cos_sin && positions && slot_mapping && k_cache && v_cache, MI355_ERR_INVALID,
-                "rope_partial_kv_write: null pointer");
+  MI355_REQUIRE(q && cos_sin && positions && slot_mapping, MI355_ERR_INVALID, "rope_partial_kv_write: null pointer");
+  MI355_REQUIRE((k && v && k_cache && v_cache) || (!k && !v && !k_cache && !v_cache), MI355_ERR_INVALID,
+                "rope_partial_kv_write: k, v and both caches go together (all null: queries only)");
   MI355_REQUIRE(num_tokens >= 0 && num_heads > 0 && num_kv_heads > 0 && head_dim > 0 && v_dim > 0 && max_pos > 0,
                 MI355_ERR_INVALID, "rope_partial_kv_write: sizes");
   MI355_REQUIRE(rot_dims >= 0 && rot_dims <= head_dim && rot_dims % 2 == 0, MI355_ERR_INVALID,
                 "rope_partial_kv_write: rot_dims %d must be even and at most head_dim %d", rot_dims, head_dim);
   MI355_REQUIRE(q_stride >= static_cast<int64_t>(num_heads) * head_dim &&
-                    k_stride >= static_cast<int64_t>(num_kv_heads) * head_dim &&
-                    v_stride >= static_cast<int64_t>(num_kv_heads) * v_dim,
+                    (k == nullptr || (k_stride >= static_cast<int64_t>(num_kv_heads) * head_dim &&
+                                      v_stride >= static_cast<int64_t>(num_kv_heads) * v_dim)),
                 MI355_ERR_INVALID, "rope_partial_kv_write: row strides shorter than the rows");
   REQ_DTYPE(dtype);
   if (num_tokens == 0) return MI355_OK;

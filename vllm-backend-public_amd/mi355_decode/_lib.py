@@ -97,6 +97,7 @@ def _load() -> ctypes.CDLL:
         "mi355_allreduce_oneshot_destroy": (I32, [P]),
         "mi355_linear_decode": (I32, [P, I64, P, I64, P, P, I32, I32, I32, I32, I32, P]),
         "mi355_embed_scale_f32": (I32, [P, P, P, I64, I32, I64, F, I32, P]),
+        "mi355_embed_scale_pos_f32": (I32, [P, P, P, P, P, I64, I32, I64, I64, F, I32, P]),
         "mi355_resid_add_f32": (I32, [P, P, P, P, I64, I32, I32, P]),
         "mi355_add_rms_norm_f32": (I32, [P, P, P, P, I32, I64, I32, F, I32, P]),
         "mi355_rms_norm_mix_f32": (I32, [P, P, P, P, P, I64, I32, F, F, I32, P]),
@@ -131,6 +132,7 @@ def _load() -> ctypes.CDLL:
         "mi355_moe_gate_up_rows": (I32, [P, P, P, P, P, I32, I32, I32, I32, I32, F, I32, P]),
         "mi355_moe_down_rows": (I32, [P, P, P, P, I32, I32, I32, I32, P]),
         "mi355_moe_silu_and_mul": (I32, [P, P, I64, I32, I32, F, I32, P]),
+        "mi355_gated_act_rows": (I32, [P, I64, P, P, I64, I64, I32, I32, F, I32, P]),
         "mi355_moe_combine": (I32, [P, P, P, P, P, P, I32, I64, I32, I32, P, I32, P, P, I64, I32, P]),
         "mi355_embed_bigram_pos_f32": (I32, [P, P, P, P, P, P, P, P, P, P, I64, I32, I64, I64, I64, I64, I32, P]),
         "mi355_prev_token_update": (I32, [P, P, P, P, I32, P]),
@@ -138,7 +140,7 @@ def _load() -> ctypes.CDLL:
         "mi355_qk_norm_kv_write": (I32, [P, I64, P, I64, P, I64, P, P, P, P, P, I64, I32, I32, I32, I32, F, I32, P]),
         "mi355_softmax_bias_attn_workspace": (I64, [I64, I32, I32, I32]),
         "mi355_softmax_bias_attn": (I32, [P, P, I64, P, P, P, I32, P, P, P, P, P, I64, I32, I64, I32, I32, I32, I32, I32,
-                                          I32, F, P, I32, P, I32, I32, P]),
+                                          I32, F, P, I32, P, I32, P, I64, I32, P]),
         "mi355_mingru_scan": (I32, [P, P, I64, I32, I32, I32, P, P, P, P, P, P, I32, I64, I32, I32, P, I32, I32, P]),
         "mi355_mingru_scan_workspace": (I64, [I32, I32, I32]),
     }
@@ -171,7 +173,7 @@ EXPORTS = ("mi355_abi_version", "mi355_last_error", "mi355_target_arch",
            "mi355_allreduce_oneshot_run", "mi355_allreduce_oneshot_run_slabs", "mi355_allreduce_oneshot_run_add_norm", "mi355_allreduce_twoshot_run_add_norm", "mi355_allreduce_oneshot_run_max_keys",
            "mi355_allreduce_oneshot_status",
            "mi355_allreduce_oneshot_status_async", "mi355_allreduce_oneshot_destroy",
-           "mi355_embed_scale_f32", "mi355_resid_add_f32", "mi355_add_rms_norm_f32", "mi355_rms_norm_mix_f32",
+           "mi355_embed_scale_f32", "mi355_embed_scale_pos_f32", "mi355_gated_act_rows", "mi355_resid_add_f32", "mi355_add_rms_norm_f32", "mi355_rms_norm_mix_f32",
            "mi355_gelu_tanh_and_mul", "mi355_gated_head_rms_norm", "mi355_softcap",
            "mi355_rope_partial_kv_write", "mi355_sigmoid_window_attn", "mi355_causal_conv_silu",
            "mi355_conv_state_update", "mi355_gated_delta_rule", "mi355_gated_delta_rule_workspace",

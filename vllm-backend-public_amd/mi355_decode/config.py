@@ -14,7 +14,7 @@ import os
 from dataclasses import dataclass, field
 from typing import Any, Optional
 
-SUPPORTED_ARCHS = ("LlamaForCausalLM", "Qwen2ForCausalLM", "MistralForCausalLM", "OPTForCausalLM", "Lozupel", "Tativik", "Tafisun")
+SUPPORTED_ARCHS = ("LlamaForCausalLM", "Qwen2ForCausalLM", "MistralForCausalLM", "OPTForCausalLM", "Lozupel", "Tativik", "Tafisun", "Bemulorn")
 
 # Well-known geometries, used when --model names one of them and no local
 # config.json exists (synthetic-weight benchmarking; there is no network).
@@ -118,7 +118,10 @@ class MoESpec:
     keep: int
     ff: int
     # what follows defaults to the first design that used this spec
-    score: str = "sigmoid"                  # "sigmoid": each expert by itself; "softmax": over all router outputs
+    score: str = "sigmoid"                  # "sigmoid": each expert by itself; "softmax": over all router outputs;
+                                            # "chosen_softmax": choice by the logits, weights a softmax over the chosen alone
+    router_bias: bool = False               # the router logits carry a learned bias
+    shared_gated: bool = True               # the shared expert is scaled by a sigmoid of one projected number per token
     group_score: str = "top2"               # a group scores the sum of its two best choice scores, or ("max") its best
     weight_scale: float = 1.0               # the chosen experts' scores are multiplied by this
     identity: int = 0                       # router outputs past `experts` that stand for "the input itself"; groups
@@ -148,7 +151,15 @@ class BlockAttnSpec:
     q.k * scale - r1[h] * ln(1 + r2[h] * (i - j)).  Queries and keys get an RMS norm per head with one
     weight vector shared by the heads.  values_are_keys: no value projection exists; the key
     projection, taken ahead of its norm, doubles as the value (then vdim == dim).  The concatenated heads are
-    multiplied by a sigmoid gate of their own width."""
+    multiplied by a sigmoid gate of their own width.
+
+    What follows the first design's fields switches its particulars off and others on: qk_norm /
+    penalty False: plain q.k * scale; rot_dims > 0: rotary positions on the first rot_dims coordinates
+    of every query and key head (coordinate i paired with i + rot_dims / 2), frequencies blended for
+    longer contexts by rot_scaling; bias: q, k and v projections carry biases; sink: the softmax
+    denominator holds one more term exp(sink) that carries no value; gate_per_head: the gate is one
+    number per head; kv_from: the layer has no key / value projections and attends to the pages of
+    that earlier layer."""
     heads: int
     kv_heads: int
     dim: int
@@ -156,6 +167,40 @@ class BlockAttnSpec:
     block: int
     scale: float
     values_are_keys: bool = True
+    qk_norm: bool = True
+    penalty: bool = True
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_scaling: Optional["RotaryScaling"] = None
+    bias: bool = False
+    sink: Optional[float] = None
+    gate_per_head: bool = False
+    kv_from: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class RotaryScaling:
+    """Blend of rotary frequencies for contexts longer than `original` positions: with
+    c(r) = dims * ln(original / (2 pi r)) / (2 ln base), lo = max(floor(c(fast)), 0),
+    hi = min(ceil(c(slow)), dims - 1) and m_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at
+    f_i / factor * m_i + f_i * (1 - m_i); cos and sin are both multiplied by 0.1 ln(factor) + 1."""
+    factor: float
+    original: float
+    fast: float
+    slow: float
+
+    def frequencies(self, rot_dims: int, base: float):
+        """(float64 frequencies [rot_dims / 2], the factor on cos and sin)."""
+        import math
+        import numpy as np
+        i = np.arange(rot_dims // 2, dtype=np.float64)
+        f = float(base) ** (-2.0 * i / rot_dims)
+
+        def c(r):
+            return rot_dims * math.log(self.original / (2.0 * math.pi * r)) / (2.0 * math.log(base))
+        lo, hi = max(math.floor(c(self.fast)), 0), min(math.ceil(c(self.slow)), rot_dims - 1)
+        m = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return f / self.factor * m + f * (1.0 - m), 0.1 * math.log(self.factor) + 1.0
 
 
 @dataclass
@@ -188,7 +233,10 @@ class HybridLayerSpec:
     moe: Optional[MoESpec] = None           # a mixture-of-experts feed-forward instead of a dense one
     battn: Optional[BlockAttnSpec] = None   # kind "attention"
     gru: Optional[MinGRUSpec] = None        # kind "mingru"
-    ff_act: str = "gelu_gated"              # the dense feed-forward: gelu_tanh(gate) * up, or "relu2": relu(up)^2, no gate
+    ff_act: str = "gelu_gated"              # the dense feed-forward: gelu_tanh(gate) * up, or "relu2": relu(up)^2, no gate,
+                                            # or "limited": g' sigmoid(1.702 g') (u' + 1), g' = min(g, ff_limit),
+                                            # u' = clamp(u, -ff_limit, ff_limit)
+    ff_limit: Optional[float] = None
 
 
 @dataclass
@@ -205,13 +253,16 @@ class HybridSpec:
     loop_times: int = 0                     # 0: no loop
     # "pre": x += sublayer(norm(x)), norms with one learned number.  "sandwich": the embedding is
     # normed, and x += residual_mult * norm_b(sublayer(h) * sigmoid(Wg h + bg)) with h = norm(x);
-    # every such norm is an RMS norm in norm_groups equal parts with a weight vector
+    # every such norm is an RMS norm in norm_groups equal parts with a weight vector.  "parallel":
+    # x += mixer(h) + ff(h) with h = norm(x): one norm per layer, both sub-layers read it
     arrangement: str = "pre"
     norm_groups: int = 1
     residual_mult: float = 1.0
     norm_vector: bool = False               # "pre" arrangement: norms carry a weight per channel instead of one number
     bigram: Optional[BigramSpec] = None     # a hashed previous-token embedding is added (the previous token is state)
     sinusoid_base: float = 0.0              # > 0: sin / cos of pos * base^(-2i / width) in entries 2i / 2i + 1 is added
+    learned_positions: bool = False         # a learned vector per position is added to the scaled embedding
+    logit_scale: float = 1.0                # the logits are multiplied by this
 
     def runs(self):
         """[(layer index, pass number or None)] in execution order: one cache / state each."""
@@ -222,6 +273,52 @@ class HybridSpec:
         for t in range(self.loop_times):
             out += [(i, t) for i in range(self.loop_start, self.loop_stop)]
         return out + [(i, None) for i in range(self.loop_stop, n)]
+
+    @classmethod
+    def from_bemulorn(cls, d: dict) -> "HybridSpec":
+        layers = []
+        for i, spec in enumerate(d["layers"]):
+            m, mlp = spec["mixer"], spec.get("mlp")
+            kw = {}
+            if mlp is not None and mlp.get("kind", "dense") == "dense":
+                kw.update(ff=int(mlp["ff"]), ff_act="limited", ff_limit=float(mlp["limit"]))
+            elif mlp is not None and mlp.get("kind") == "moe":
+                r, sh = mlp["router"], mlp.get("shared") or None
+                moe = MoESpec(experts=int(r["experts"]), top=int(r["top"]), groups=1, keep=1, ff=int(mlp["expert"]["ff"]),
+                              score="chosen_softmax", router_bias=True, shared_ff=int(sh["ff"]) if sh else 0,
+                              shared_gated=False)
+                moe.check(f"layer {i}")
+                kw.update(moe=moe)
+            elif mlp is not None:
+                raise ValueError(f"feed-forward kind {mlp.get('kind')!r} is not supported (dense, moe)")
+            if spec["type"] != "attention":
+                raise ValueError(f"layer type {spec['type']!r} is not supported (attention)")
+            rot = m.get("rot") or {}
+            sc = rot.get("scaling") or None
+            a = BlockAttnSpec(heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]),
+                              vdim=int(m.get("vdim", m["dim"])), block=int((m.get("mask") or {}).get("size") or 0),
+                              scale=float(m["scale"]), values_are_keys=False, qk_norm=False, penalty=False,
+                              rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)),
+                              rot_scaling=RotaryScaling(float(sc["factor"]), float(sc["original"]), float(sc["fast"]),
+                                                        float(sc["slow"])) if sc else None,
+                              bias=True, sink=0.0, gate_per_head=True,
+                              kv_from=(int(m["kv_from"]) if m.get("kv_from") is not None else None))
+            if a.heads < 1 or a.kv_heads < 1 or a.heads % a.kv_heads:
+                raise ValueError(f"layer {i}: kv_heads {a.kv_heads} must divide heads {a.heads}")
+            if a.rot_dims > a.dim or a.rot_dims % 2:
+                raise ValueError(f"layer {i}: {a.rot_dims} rotated coordinates do not fit heads of {a.dim}")
+            if a.kv_from is not None:
+                src = layers[a.kv_from].battn if 0 <= a.kv_from < i else None
+                if src is None or src.kv_from is not None:
+                    raise ValueError(f"layer {i}: kv_from {a.kv_from} must name an earlier attention layer that has "
+                                     "key and value projections of its own")
+                if (src.kv_heads, src.dim, src.vdim, src.rot_dims, src.rot_base, src.rot_scaling) != \
+                        (a.kv_heads, a.dim, a.vdim, a.rot_dims, a.rot_base, a.rot_scaling):
+                    raise ValueError(f"layer {i}: key / value heads and rotation differ from layer {a.kv_from}'s")
+            layers.append(HybridLayerSpec("attention", battn=a, **kw))
+        return cls(layers=layers, arrangement="parallel", norm_vector=True, learned_positions=True,
+                   embed_scale=float((d.get("embedding") or {}).get("scale", 1.0)),
+                   logit_scale=float(d.get("logit_scale", 1.0)))
 
     @classmethod
     def from_tafisun(cls, d: dict) -> "HybridSpec":
@@ -393,6 +490,19 @@ class ModelConfig:
                    eos_token_id=d.get("eos_token_id"), family="hybrid", hybrid=spec)
 
     @classmethod
+    def _from_bemulorn_dict(cls, d: dict) -> "ModelConfig":
+        spec = HybridSpec.from_bemulorn(d)
+        att = [L.battn for L in spec.layers]
+        ffs = [L.ff or 0 for L in spec.layers] + [max(L.moe.ff, L.moe.shared_ff) for L in spec.layers if L.moe] + [0]
+        return cls(architecture="Bemulorn", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]),
+                   intermediate_size=max(ffs), num_hidden_layers=len(spec.layers),
+                   num_attention_heads=max([a.heads for a in att] + [1]), num_key_value_heads=max([a.kv_heads for a in att] + [1]),
+                   head_dim=max([a.dim for a in att] + [1]), rope_theta=0.0, rope_scaling=None,
+                   rms_norm_eps=float(d["norm"]["eps"]), max_position_embeddings=int(d.get("max_positions", 1 << 17)),
+                   tie_word_embeddings=False, attention_bias=True, bos_token_id=d.get("bos_token_id"),
+                   eos_token_id=d.get("eos_token_id"), family="hybrid", hybrid=spec)
+
+    @classmethod
     def _from_tativik_dict(cls, d: dict) -> "ModelConfig":
         spec = HybridSpec.from_tativik(d)
         if int(d["width"]) % spec.norm_groups:
@@ -441,9 +551,9 @@ class ModelConfig:
             cfg = cls._from_opt_dict(d)
             cfg.torch_dtype = stored
             return cfg
-        if arch in ("Lozupel", "Tativik", "Tafisun"):
+        if arch in ("Lozupel", "Tativik", "Tafisun", "Bemulorn"):
             cfg = {"Lozupel": cls._from_lozupel_dict, "Tativik": cls._from_tativik_dict,
-                   "Tafisun": cls._from_tafisun_dict}[arch](d)
+                   "Tafisun": cls._from_tafisun_dict, "Bemulorn": cls._from_bemulorn_dict}[arch](d)
             cfg.torch_dtype = stored or "bfloat16"
             return cfg
         nh = d["num_attention_heads"]

@@ -11,7 +11,14 @@ mixer and may carry a feed-forward.  Two arrangements share this runner:
   * "sandwich" (the Tativik design): a general delta rule (decay per key channel, removal along the
     unit key) or a softmax attention through low-rank latents (sliding window, a sink in the
     denominator, latent pages that a later layer may share), then a mixture of experts; every
-    sub-layer sits between a norm in groups and a gated, normed, scaled residual add.
+    sub-layer sits between a norm in groups and a gated, normed, scaled residual add;
+  * "parallel" (the Bemulorn design): one norm per layer whose output both sub-layers read,
+    x += attention(h) + ff(h); learned positions beside a scaled embedding; the attention is the
+    block attention without norms and penalty but with biased projections, rotary positions on part
+    of every head (frequencies blended for long contexts), a value-less term in the softmax
+    denominator, one gate per head and key / value pages that a later layer may share; the
+    feed-forward is a limited gated unit or a mixture whose weights are a softmax over the chosen
+    logits, plus an ungated shared expert.
 
 What differs from ModelRunner's decoders, and where it lives:
   * the residual stream is float32 (csrc/resid32.hip: norms with one learned number or a vector,
@@ -42,12 +49,19 @@ from .model_runner import ModelRunner, batch_buckets
 from .weights import ModelWeights
 
 
-def rotary_table(rot_dims: int, base: float, max_pos: int, device) -> torch.Tensor:
-    """float32 [max_pos, rot_dims] = cos | sin of pos * base^(-2i / rot_dims), i < rot_dims / 2."""
+def rotary_table(rot_dims: int, base: float, max_pos: int, device, scaling=None) -> torch.Tensor:
+    """float32 [max_pos, rot_dims] = cos | sin of pos * base^(-2i / rot_dims), i < rot_dims / 2.
+    scaling (config.RotaryScaling): its blended frequencies instead, cos and sin times its factor.
+    Angles are formed in float32 from float32 frequencies."""
     half = rot_dims // 2
-    inv = float(base) ** (-2.0 * torch.arange(half, dtype=torch.float32, device=device) / rot_dims)
+    mult = 1.0
+    if scaling is None:
+        inv = float(base) ** (-2.0 * torch.arange(half, dtype=torch.float32, device=device) / rot_dims)
+    else:
+        f, mult = scaling.frequencies(rot_dims, base)
+        inv = torch.from_numpy(f.astype(np.float32)).to(device)
     ang = torch.arange(max_pos, dtype=torch.float32, device=device)[:, None] * inv[None, :]
-    return torch.cat([ang.cos(), ang.sin()], dim=1).contiguous()
+    return (torch.cat([ang.cos(), ang.sin()], dim=1) * mult).contiguous()
 
 
 class StepBatch:
@@ -183,6 +197,32 @@ class BlockAttention:
         return r.linear(o, lw.o_w)
 
 
+class RotaryBlockAttention:
+    """Softmax attention inside blocks of positions over the paged K/V of one layer run -- its own
+    (it writes them first) or those of the layer it shares with: biased projections, rotary positions
+    on the first rot_dims coordinates of every head, one more value-less term in the softmax
+    denominator, one sigmoid gate per head.  Writes the gated heads into `out`, a column slice of
+    the row that the layer's output matrix multiplies."""
+
+    def __init__(self, spec, lw, runner, cache_index: int, writes: bool):
+        self.s, self.lw, self.r, self.ci, self.writes = spec, lw, runner, cache_index, writes
+
+    def __call__(self, proj: torch.Tensor, b: StepBatch, out: torch.Tensor) -> torch.Tensor:
+        s, lw, r = self.s, self.lw, self.r
+        col = lambda n: proj[:, lw.seg[n][0]: lw.seg[n][0] + lw.seg[n][1]]     # noqa: E731
+        q = col("q")
+        kc, vc = r.k_cache[self.ci], r.v_cache[self.ci]
+        table = r.rotary(s.rot_dims, s.rot_base, s.rot_scaling)
+        if self.writes:
+            ops.rope_partial_kv_write(q, col("k"), col("v"), table, b.positions, b.slot_mapping, kc, vc, s.heads, s.kv_heads,
+                                      s.dim, s.vdim)
+        elif s.rot_dims > 0:
+            ops.rope_partial_kv_write(q, None, None, table, b.positions, b.slot_mapping, None, None, s.heads, s.kv_heads,
+                                      s.dim, s.vdim)
+        return ops.softmax_bias_attn(q, kc, vc, b.block_tables, b.tok_seq, b.positions, None, None, col("g"), s.heads, s.scale,
+                                     block=s.block, tiles=b.tiles, num_splits=r.block_key_splits(b, s), sink=lw.sink, out=out)
+
+
 class MinGRUMixer:
     """Per-channel gated recurrence on one layer run's state slots: gates and candidate from the
     current token only, the state in float32."""
@@ -218,16 +258,19 @@ class MoEFeedForward:
 
     GROUPED_MAX_TOKENS = 2048       # longer steps go through the experts in slices of this many tokens
 
-    def __call__(self, h: torch.Tensor) -> torch.Tensor:
+    def __call__(self, h: torch.Tensor, shared: Optional[torch.Tensor] = None) -> torch.Tensor:
         """h [tokens, width] -> the mixture's output, the same shape.  Tokens are independent of each other
         here, so a long step is served in slices: the padded batched products then stay at sizes where
-        an uneven slice costs little padding, and their temporaries at a few hundred megabytes."""
+        an uneven slice costs little padding, and their temporaries at a few hundred megabytes.
+        shared [tokens, width]: rows the caller has computed already (a shared expert, another
+        sub-layer's output) that the weighted sum takes in unscaled, instead of a shared expert run here."""
         T = h.shape[0]
         if T <= self.GROUPED_MAX_TOKENS:
-            return self._tokens(h)
+            return self._tokens(h, shared)
         out = torch.empty_like(h)
         for a in range(0, T, self.GROUPED_MAX_TOKENS):
-            out[a: a + self.GROUPED_MAX_TOKENS] = self._tokens(h[a: a + self.GROUPED_MAX_TOKENS])
+            out[a: a + self.GROUPED_MAX_TOKENS] = self._tokens(h[a: a + self.GROUPED_MAX_TOKENS],
+                                                               None if shared is None else shared[a: a + self.GROUPED_MAX_TOKENS])
         return out
 
     def _act(self, gu: torch.Tensor, limit, ff: int) -> torch.Tensor:
@@ -235,21 +278,28 @@ class MoEFeedForward:
             return ops.silu_and_mul(gu)
         return ops.moe_silu_and_mul(gu, limit)
 
-    def _tokens(self, h: torch.Tensor) -> torch.Tensor:
+    def _tokens(self, h: torch.Tensor, shared: Optional[torch.Tensor] = None) -> torch.Tensor:
         s, lw = self.s, self.lw
         T, E = h.shape[0], s.experts
         # the router product in fp32; a shared expert's gate is one more row of the same matrix
-        logits = torch.mm(h.float(), lw.router_w.t())
+        if s.router_bias:
+            logits = torch.addmm(lw.router_b, h.float(), lw.router_w.t())
+        else:
+            logits = torch.mm(h.float(), lw.router_w.t())
         ids, wts = ops.moe_route(logits, lw.correction, s.top, s.groups, s.keep, softmax=s.score == "softmax",
-                                 group_max=s.group_score == "max", weight_scale=s.weight_scale, experts=s.outputs)
+                                 group_max=s.group_score == "max", weight_scale=s.weight_scale, experts=s.outputs,
+                                 chosen_softmax=s.score == "chosen_softmax")
         offsets, perm, inv = ops.moe_sort(ids, s.outputs)
         extra = {}
         if s.identity:
             extra.update(ids=ids, x=h, num_real=E)
-        if s.shared_ff:
+        if shared is not None:
+            extra.update(shared=shared.contiguous())
+        elif s.shared_ff:
             gu = self.r.linear(h, lw.shared_gate_up_w)
-            extra.update(shared=self.r.linear(self._act(gu, s.shared_limit, s.shared_ff), lw.shared_down_w),
-                         shared_gate=logits[:, s.outputs:])
+            extra.update(shared=self.r.linear(self._act(gu, s.shared_limit, s.shared_ff), lw.shared_down_w))
+            if s.shared_gated:
+                extra.update(shared_gate=logits[:, s.outputs:])
         rows = T * s.top
         if rows >= self.GROUPED_MIN_ROWS and not torch.cuda.is_current_stream_capturing():
             # many rows: library GEMMs per expert.  The experts' row ranges come to the host (one wait); when
@@ -339,7 +389,18 @@ class HybridRunner(ModelRunner):
                 self.mixers.append(LatentAttention(A, lw, self, latent_of[li if A.kv_from is None else A.kv_from],
                                                    A.kv_from is None))
             self.ffs.append(MoEFeedForward(L.moe, lw, self) if L.moe is not None else None)
-        for li, _ in self.runs if spec.arrangement != "sandwich" else ():
+        pages_of = {}                                   # layer index -> index of its K/V pages
+        for li, _ in self.runs if spec.arrangement == "parallel" else ():
+            L, lw = spec.layers[li], weights.layers[li]
+            A = L.battn
+            if A.kv_from is None:
+                self.k_cache.append(torch.zeros(self.num_blocks, A.kv_heads, BLOCK_SIZE, A.dim, dtype=dtype, device=dev))
+                self.v_cache.append(torch.zeros(self.num_blocks, A.kv_heads, A.vdim, BLOCK_SIZE, dtype=dtype, device=dev))
+                pages_of[li] = len(self.k_cache) - 1
+            self.mixers.append(RotaryBlockAttention(A, lw, self, pages_of[li if A.kv_from is None else A.kv_from],
+                                                    A.kv_from is None))
+            self.ffs.append(MoEFeedForward(L.moe, lw, self) if L.moe is not None else None)
+        for li, _ in self.runs if spec.arrangement == "pre" else ():
             L, lw = spec.layers[li], weights.layers[li]
             self.ffs.append(MoEFeedForward(L.moe, lw, self) if L.moe is not None else
                             ReluSquaredFF(lw, self) if L.ff and L.ff_act == "relu2" else None)
@@ -380,7 +441,8 @@ class HybridRunner(ModelRunner):
         # the samplers want 16-byte aligned logit rows: the head is padded with zero rows to a multiple
         # of 8 and the logits are the first V columns of what it yields
         self.Vp = -(-self.V // 8) * 8
-        self._forward = self._forward_sandwich if spec.arrangement == "sandwich" else self._forward_pre
+        self._forward = {"sandwich": self._forward_sandwich, "parallel": self._forward_parallel}.get(spec.arrangement,
+                                                                                                     self._forward_pre)
         self.head_w = weights.lm_head
         if self.Vp != self.V:
             self.head_w = torch.zeros(self.Vp, self.H, dtype=dtype, device=dev)
@@ -403,10 +465,10 @@ class HybridRunner(ModelRunner):
         self._dec_pairs = {}                          # of a decode step of max_num_seqs rows: heads -> device tiles
 
     # ------------------------------------------------------------------ #
-    def rotary(self, rot_dims: int, base: float) -> torch.Tensor:
-        key = (rot_dims, base)
+    def rotary(self, rot_dims: int, base: float, scaling=None) -> torch.Tensor:
+        key = (rot_dims, base, scaling)
         if key not in self._rotary:
-            self._rotary[key] = rotary_table(rot_dims, base, self.max_blocks * BLOCK_SIZE, self.device)
+            self._rotary[key] = rotary_table(rot_dims, base, self.max_blocks * BLOCK_SIZE, self.device, scaling)
         return self._rotary[key]
 
     def _decode_pair_tiles(self, heads: int) -> torch.Tensor:
@@ -471,14 +533,16 @@ class HybridRunner(ModelRunner):
         mats = [self.head_w]
         for lw in self.w.layers:
             mats += [getattr(lw, n, None) for n in ("in_w", "delta_o_w", "attn_o_w", "gate_up_w", "down_w", "a2_w", "g2_w",
-                                                    "o_w", "uq_w", "w2_w", "rg2_w", "up_w", "shared_gate_up_w", "shared_down_w")]
+                                                    "o_w", "uq_w", "w2_w", "rg2_w", "up_w", "shared_gate_up_w", "shared_down_w",
+                                                    "out_w")]
         for w in mats:
             # the kernel stages x in 512-wide K slices; narrow outputs leave too few workgroups to pay
             if w is not None and w.dim() == 2 and w.shape[1] % 512 == 0 and w.shape[0] >= 256 and w.shape[0] % 8 == 0:
                 self._tiled_w[w.data_ptr()] = ops.tile_weights(w)
 
-    def linear(self, x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """x @ w.T.  Decode-sized row counts stream the weights once: through the fragment-tiled copy
+    def linear(self, x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None,
+               bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x @ w.T (+ bias, in the accumulator's float32 ahead of the rounding).  Decode-sized row counts stream the weights once: through the fragment-tiled copy
         (K split over workgroups into fp32 slabs where one pass would leave most of the chip idle, a
         second launch adds the slabs) or, for matrices that have none, row-major through
         mi355_linear_decode.  A library GEMM otherwise (prefill; float32; odd widths)."""
@@ -493,11 +557,13 @@ class HybridRunner(ModelRunner):
                 if out is None:
                     out = torch.empty(M, N, dtype=x.dtype, device=x.device)
                 if groups == 1:
-                    return ops.linear_tiled(x, tw, N, out=out, tiles_per_wg=tiles)
+                    return ops.linear_tiled(x, tw, N, bias=bias, out=out, tiles_per_wg=tiles)
                 part = ops.linear_tiled(x, tw, N, tiles_per_wg=tiles, k_groups=groups, epilogue=ops.EPI_PARTIAL)
-                return ops.sum_slabs(part, groups, out)
+                return ops.sum_slabs(part, groups, out, bias=bias)
         if ok16 and M <= ops.LINEAR_DECODE_MAX_M and K % 32 == 0 and N % 4 == 0:
-            return ops.linear_decode(x, w, None, out=out)
+            return ops.linear_decode(x, w, bias, out=out)
+        if bias is not None:
+            return torch.addmm(bias, x, w.t()) if out is None else torch.addmm(bias, x, w.t(), out=out)
         if out is None:
             return torch.mm(x, w.t())
         return torch.mm(x, w.t(), out=out)
@@ -589,6 +655,41 @@ class HybridRunner(ModelRunner):
                 self.layer_trace.append(resid.clone())
         return resid
 
+    def _forward_parallel(self, b: StepBatch) -> torch.Tensor:
+        """All layers of the parallel arrangement over one packed batch; returns the float32 residual
+        stream [tokens, width].  Per layer: one norm (the previous layer's output rides in its launch),
+        one product for everything that reads it, the attention and the gated activation writing side by
+        side into one row, one product back: the sum of both sub-layers."""
+        w, spec = self.w, self.spec
+        if spec.learned_positions:
+            resid = ops.embed_scale_pos_f32(w.embed, b.ids, spec.embed_scale, w.pos_embed, b.positions)
+        else:
+            resid = ops.embed_scale_f32(w.embed, b.ids, spec.embed_scale)
+        T, pending, last = b.num_tokens, None, len(self.runs) - 1
+        for ri, (li, _) in enumerate(self.runs):
+            L, lw = spec.layers[li], w.layers[li]
+            A = L.battn
+            h = ops.add_rms_norm_f32(resid, lw.norm1, self.eps, add=pending)
+            proj = self.linear(h, lw.in_w, bias=lw.in_b)
+            n_attn = A.heads * A.vdim
+            at, K = -(-n_attn // 8) * 8, lw.out_w.shape[1]          # the hidden units start on a 16-byte boundary
+            row = (torch.zeros if at != n_attn else torch.empty)(T, K, dtype=self.dtype, device=self.device)
+            self.mixers[ri](proj, b, row[:, :n_attn])
+            if K > at:
+                seg = lw.seg
+                ops.gated_act_rows(proj[:, seg["gate"][0]: seg["gate"][0] + seg["gate"][1]],
+                                   proj[:, seg["up"][0]: seg["up"][0] + seg["up"][1]],
+                                   L.ff_limit if L.ff else L.moe.shared_limit, out=row[:, at:])
+            pending = self.linear(row, lw.out_w)
+            if self.ffs[ri] is not None:
+                pending = self.ffs[ri](h, shared=pending)
+            if ri == last or self.layer_trace is not None:
+                ops.resid_add_f32(resid, rows=pending)
+                pending = None
+            if self.layer_trace is not None:
+                self.layer_trace.append(resid.clone())
+        return resid
+
     def _logits(self, resid: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Final norm, head and soft cap over the given residual rows."""
         if self.spec.arrangement == "sandwich":
@@ -598,6 +699,8 @@ class HybridRunner(ModelRunner):
         z = self.linear(h, self.head_w, out=out)
         if self.spec.logit_softcap:
             ops.softcap(z, self.spec.logit_softcap)
+        if self.spec.logit_scale != 1.0:
+            z.mul_(self.spec.logit_scale)
         return z[:, : self.V]
 
     # ------------------------------------------------------------------ #

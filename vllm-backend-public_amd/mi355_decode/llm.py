@@ -62,7 +62,8 @@ def plan_num_blocks(args: EngineArgs, cfg: ModelConfig, tp_size: int, num_layers
     per_block = 2 * num_layers * (cfg.num_key_value_heads // tp_size) * BLOCK_SIZE * cfg.head_dim * elem_size
     if cfg.family == "hybrid":                        # K and V pages of every layer run that has an attention
         runs = [cfg.hybrid.layers[i] for i, _ in cfg.hybrid.runs()]
-        per_tok = sum(a.kv_heads * (a.dim + a.vdim) for L in runs for a in (L.attn, L.battn) if a is not None)
+        per_tok = sum(a.kv_heads * (a.dim + a.vdim) for L in runs for a in (L.attn, L.battn)
+                      if a is not None and getattr(a, "kv_from", None) is None)    # (a layer may read another layer's pages)
         # a latent attention caches its latent and one rotated key part, unless it reads another layer's
         # (in 16 bits the latent twice: token-major for the scores, channel-major for the weighted sum)
         per_tok += sum((1 if elem_size == 4 else 2) * L.lattn.kv_rank + L.lattn.rot_dim for L in runs
@@ -103,6 +104,10 @@ def build_engine(args: EngineArgs, state_dict: Optional[dict] = None, model_conf
                     args.block_size, BLOCK_SIZE)
     max_model_len = args.max_model_len or min(cfg.max_position_embeddings, 8192)
     if cfg.family == "opt" and max_model_len > cfg.max_position_embeddings:
+        log.warning("--max-model-len %d exceeds the model's %d learned positions: serving %d", max_model_len,
+                    cfg.max_position_embeddings, cfg.max_position_embeddings)
+        max_model_len = cfg.max_position_embeddings
+    if cfg.family == "hybrid" and cfg.hybrid.learned_positions and max_model_len > cfg.max_position_embeddings:
         log.warning("--max-model-len %d exceeds the model's %d learned positions: serving %d", max_model_len,
                     cfg.max_position_embeddings, cfg.max_position_embeddings)
         max_model_len = cfg.max_position_embeddings

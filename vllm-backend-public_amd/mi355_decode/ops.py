@@ -964,6 +964,22 @@ def embed_scale_f32(embed: torch.Tensor, ids: torch.Tensor, scale: float, out: t
     return out
 
 
+def embed_scale_pos_f32(embed: torch.Tensor, ids: torch.Tensor, scale: float, pos_table: torch.Tensor,
+                        positions: torch.Tensor):
+    """float32 rows embed[ids[t]] * scale + pos_table[positions[t]] (learned positions, unscaled)."""
+    dt = _dt3(embed, "embed")
+    if embed.dim() != 2 or not embed.is_contiguous():
+        raise ValueError("embed must be contiguous [vocab, width]")
+    T, W = ids.numel(), embed.shape[1]
+    if pos_table.dtype != embed.dtype or pos_table.dim() != 2 or pos_table.shape[1] != W or not pos_table.is_contiguous():
+        raise ValueError("pos_table must be contiguous [positions, width] in the dtype of embed")
+    out = torch.empty(T, W, dtype=torch.float32, device=embed.device)
+    check(lib.mi355_embed_scale_pos_f32(out.data_ptr(), embed.data_ptr(), pos_table.data_ptr(), _idx(ids, "ids", torch.int64),
+                                        _idx(positions, "positions", torch.int64, T), T, W, embed.shape[0],
+                                        pos_table.shape[0], float(scale), dt, _stream()))
+    return out
+
+
 def resid_add_f32(resid: torch.Tensor, other: torch.Tensor | None = None, rows: torch.Tensor | None = None,
                   vec: torch.Tensor | None = None):
     """resid (float32, in place) += other (float32 rows) + rows (activation rows) + vec (one row)."""
@@ -1066,14 +1082,24 @@ def _cols(t: torch.Tensor, name: str, width: int) -> int:
     return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), width)
 
 
-def rope_partial_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos_sin: torch.Tensor,
-                          positions: torch.Tensor, slot_mapping: torch.Tensor, k_cache: torch.Tensor,
-                          v_cache: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, v_dim: int):
+def rope_partial_kv_write(q: torch.Tensor, k: torch.Tensor | None, v: torch.Tensor | None, cos_sin: torch.Tensor,
+                          positions: torch.Tensor, slot_mapping: torch.Tensor, k_cache: torch.Tensor | None,
+                          v_cache: torch.Tensor | None, num_heads: int, num_kv_heads: int, head_dim: int, v_dim: int):
     """Rotates q in place and k into its page by the float32 table cos_sin [max_pos, rot_dims]; copies v
-    into its page.  q / k / v may be column slices of one projection output."""
+    into its page.  q / k / v may be column slices of one projection output.  k, v and the caches None:
+    only q is rotated (a layer that attends to another layer's pages)."""
     dt = _dt3(q, "q")
     T = q.shape[0]
     rot = cos_sin.shape[1]
+    if k is None:
+        if v is not None or k_cache is not None or v_cache is not None:
+            raise ValueError("k, v and both caches go together")
+        check(lib.mi355_rope_partial_kv_write(
+            q.data_ptr(), _cols(q, "q", num_heads * head_dim), None, 0, None, 0, _f32(cos_sin, "cos_sin") or q.data_ptr(),
+            max(cos_sin.shape[0], 1), _idx(positions, "positions", torch.int64, T),
+            _idx(slot_mapping, "slot_mapping", torch.int64, T), None, None, T, num_heads, num_kv_heads, head_dim, v_dim,
+            rot, dt, _stream()))
+        return
     if tuple(k_cache.shape[1:]) != (num_kv_heads, BLOCK_SIZE, head_dim) or tuple(v_cache.shape[1:]) != (num_kv_heads, v_dim, BLOCK_SIZE) \
             or k_cache.shape[0] != v_cache.shape[0] or not k_cache.is_contiguous() or not v_cache.is_contiguous():
         raise ValueError("K pages must be [blocks, kv_heads, 16, head_dim] and V pages [blocks, kv_heads, v_dim, 16]")
@@ -1394,11 +1420,12 @@ def latent_window_attn(q_latent: torch.Tensor, q: torch.Tensor, q_head_width: in
 
 
 def moe_route(logits: torch.Tensor, correction: torch.Tensor, top: int, groups: int, keep: int, softmax: bool = False,
-              group_max: bool = False, weight_scale: float = 1.0, experts: int | None = None):
+              group_max: bool = False, weight_scale: float = 1.0, experts: int | None = None, chosen_softmax: bool = False):
     """float32 router logits [tokens, >= experts] (rows may carry more columns than router outputs:
     `experts` says how many count) -> (ids int32 [tokens, top], weights float32 [tokens, top]).
     Scores are a sigmoid per logit or (softmax) a softmax over the router outputs; a group scores the
-    sum of its two best choice scores or (group_max) its best."""
+    sum of its two best choice scores or (group_max) its best.  chosen_softmax: the choice is by the
+    logits themselves and the weights are a softmax over the chosen logits alone."""
     T = logits.shape[0]
     E = int(experts) if experts is not None else logits.shape[1]
     _dev(logits, "logits")
@@ -1407,7 +1434,8 @@ def moe_route(logits: torch.Tensor, correction: torch.Tensor, top: int, groups: 
     ids = torch.empty(T, top, dtype=torch.int32, device=logits.device)
     wts = torch.empty(T, top, dtype=torch.float32, device=logits.device)
     check(lib.mi355_moe_route(ids.data_ptr(), wts.data_ptr(), logits.data_ptr(), logits.stride(0) if T > 1 else logits.shape[1],
-                              _f32(correction, "correction", E), T, E, int(top), int(groups), int(keep), int(bool(softmax)),
+                              _f32(correction, "correction", E), T, E, int(top), int(groups), int(keep),
+                              2 if chosen_softmax else int(bool(softmax)),
                               int(bool(group_max)), float(weight_scale), _stream()))
     return ids, wts
 
@@ -1483,6 +1511,24 @@ def moe_silu_and_mul(x: torch.Tensor, limit: float | None = None):
     out = torch.empty(x.shape[0], x.shape[1] // 2, dtype=x.dtype, device=x.device)
     fn, lim = _gate_act(limit)
     check(lib.mi355_moe_silu_and_mul(out.data_ptr(), x.data_ptr(), x.shape[0], x.shape[1] // 2, fn, lim, dt, _stream()))
+    return out
+
+
+def gated_act_rows(gate: torch.Tensor, up: torch.Tensor, limit: float | None = None, out: torch.Tensor | None = None):
+    """a(gate, up) (see moe_gate_up_rows) for [rows, ff] column slices of one buffer (equal row
+    strides), into `out` [rows, ff], which may be a column slice of a wider buffer."""
+    dt = _dt3(gate, "gate")
+    R, F = gate.shape
+    if up.shape != gate.shape or up.dtype != gate.dtype or gate.stride(1) != 1 or up.stride(1) != 1 \
+            or (R > 1 and gate.stride(0) != up.stride(0)):
+        raise ValueError("gate and up must be [rows, ff] slices with equal row strides and contiguous columns")
+    if out is None:
+        out = torch.empty(R, F, dtype=gate.dtype, device=gate.device)
+    if out.shape != gate.shape or out.dtype != gate.dtype or out.stride(1) != 1:
+        raise ValueError("out must be [rows, ff] with contiguous columns in the dtype of gate")
+    fn, lim = _gate_act(limit)
+    check(lib.mi355_gated_act_rows(out.data_ptr(), _cols(out, "out", F), gate.data_ptr(), up.data_ptr(), _cols(gate, "gate", F),
+                                   R, F, fn, lim, dt, _stream()))
     return out
 
 
@@ -1590,13 +1636,16 @@ def qk_norm_kv_write(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_weight
 def softmax_bias_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                       tok_seq: torch.Tensor, positions: torch.Tensor, r1: torch.Tensor | None, r2: torch.Tensor | None,
                       gate: torch.Tensor | None, num_heads: int, scale: float, block: int = 0, window: int = 0,
-                      tiles: torch.Tensor | None = None, num_splits: int = 0):
+                      tiles: torch.Tensor | None = None, num_splits: int = 0, sink: torch.Tensor | None = None,
+                      out: torch.Tensor | None = None):
     """Softmax attention over the paged K/V [blocks, kv_heads, 16, dim] / [blocks, kv_heads, vdim, 16] with
     the score q.k * scale - r1[h] ln(1 + r2[h] * distance); a row at position p sees the keys j <= p of
     its block of `block` positions (0: all) and, window > 0, the last `window` of them.  gate
     [tokens, heads] or [tokens, heads * vdim]: the output is multiplied by its sigmoid.  tiles
     (query_tiles) selects the matrix-core form where the sizes allow; num_splits > 1 spreads a
-    tile's keys over that many workgroups.  Returns [tokens, heads * vdim]."""
+    tile's keys over that many workgroups.  sink (float32 [heads]): the softmax denominator holds one
+    more term exp(sink[h]) without a value.  out: [tokens, heads * vdim], may be a column slice of a
+    wider buffer.  Returns [tokens, heads * vdim]."""
     dt = _dt3(q, "q")
     T = q.shape[0]
     G, d, dv = k_cache.shape[1], k_cache.shape[3], v_cache.shape[2]
@@ -1605,7 +1654,10 @@ def softmax_bias_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         raise ValueError("k_cache [blocks, kv_heads, 16, dim] and v_cache [blocks, kv_heads, vdim, 16], contiguous")
     if block_tables.dim() != 2 or not block_tables.is_contiguous():
         raise ValueError("block_tables must be contiguous [chunks, max_blocks]")
-    out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
+    elif out.dtype != q.dtype or tuple(out.shape) != (T, num_heads * dv) or out.stride(1) != 1:
+        raise ValueError("out must be [tokens, heads * vdim] with contiguous columns in the dtype of q")
     per_channel, gs = 0, 0
     if gate is not None:
         per_channel = int(gate.shape[1] == num_heads * dv and dv > 1)
@@ -1621,7 +1673,8 @@ def softmax_bias_attn(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         None if r2 is None else _f32(r2, "r2", num_heads), None if gate is None else _same(gate, q, "gate"), gs, per_channel,
         T, num_heads, G, d, dv, int(block), int(window), float(scale),
         None if tiles is None else _idx(tiles, "tiles", torch.int32), 0 if tiles is None else tiles.shape[0],
-        None if ws is None else ws.data_ptr(), n, dt, _stream()))
+        None if ws is None else ws.data_ptr(), n, None if sink is None else _f32(sink, "sink", num_heads),
+        _cols(out, "out", num_heads * dv), dt, _stream()))
     return out
 
 

@@ -179,6 +179,35 @@ class MixerLayerWeights:
 
 
 @dataclass
+class ParallelLayerWeights:
+    """One layer of a hybrid decoder in the "parallel" arrangement (one norm; the attention and the
+    feed-forward both read it and their outputs are added).  Everything that reads the normed input
+    in the activation type is ONE matrix in_w with one bias row in_b (zeros where a projection has
+    none; None if no segment has one); segments `seg`: name -> (first column, width):
+      q | [k | v] | g | [gate | up of the dense feed-forward or of the shared expert]
+    (k and v are absent in a layer that attends to another layer's pages).  The two matrices that
+    lead back to the residual are one as well, side by side along their inputs:
+      out_w = [o | down]  [width, heads * vdim + ff]     (down: the dense or the shared expert's; absent: o alone)
+    so that one product over the row [attention heads | activated hidden units] yields the sum of
+    both sub-layers.  A mixture's router is float32 (router_w, router_b); its expert matrices are
+    stacked."""
+    norm1: torch.Tensor
+    in_w: torch.Tensor
+    in_b: Optional[torch.Tensor]
+    seg: dict
+    out_w: torch.Tensor
+    sink: Optional[torch.Tensor] = None         # f32 [heads]: the score of the value-less term of the softmax denominator
+    router_w: Optional[torch.Tensor] = None     # f32 [experts, width]
+    router_b: Optional[torch.Tensor] = None     # f32 [experts]
+    correction: Optional[torch.Tensor] = None   # f32 [experts], zeros: the choice is by the logits alone
+    gate_up_w: Optional[torch.Tensor] = None    # [experts, 2 ff, width]
+    down_w: Optional[torch.Tensor] = None       # [experts, width, ff]
+
+    def tensors(self):
+        return [t for t in vars(self).values() if isinstance(t, torch.Tensor)]
+
+
+@dataclass
 class ModelWeights:
     embed: torch.Tensor
     layers: list = field(default_factory=list)
@@ -200,7 +229,8 @@ class ModelWeights:
             if t is not None:
                 total += t.numel() * t.element_size()
         for lw in self.layers:
-            ts = lw.tensors() if isinstance(lw, (OPTLayerWeights, HybridLayerWeights, SandwichLayerWeights, MixerLayerWeights)) else \
+            ts = lw.tensors() if isinstance(lw, (OPTLayerWeights, HybridLayerWeights, SandwichLayerWeights, MixerLayerWeights,
+                                                 ParallelLayerWeights)) else \
                 (lw.qkv_w, lw.qkv_b, lw.o_w, lw.gate_up_w, lw.down_w, lw.input_norm, lw.post_norm)
             for t in ts:
                 if t is not None:
@@ -358,6 +388,8 @@ def _hybrid_from_getter(cfg: ModelConfig, get, dtype, device, tp_size: int, num_
         return _sandwich_from_getter(cfg, get, dtype, device)
     if cfg.architecture == "Tafisun":
         return _tafisun_from_getter(cfg, get, dtype, device)
+    if spec.arrangement == "parallel":
+        return _bemulorn_from_getter(cfg, get, dtype, device)
 
     def put(t, dt=dtype):
         return t.to(dt).contiguous().to(device)
@@ -571,6 +603,112 @@ def _tafisun_from_getter(cfg: ModelConfig, get, dtype, device) -> ModelWeights:
     return w
 
 
+def _bemulorn_from_getter(cfg: ModelConfig, get, dtype, device) -> ModelWeights:
+    """Bemulorn checkpoints: 'embed', 'pos', 'final.norm', 'head', and per layer i 'l<i>.norm1',
+    'l<i>.mix.q|k|v' with '.b', 'l<i>.mix.g|o' (no k, v in a layer that reads another layer's pages),
+    'l<i>.mlp.gate|up|down' (dense) or 'l<i>.mlp.router' with '.b', 'l<i>.mlp.e<j>.gate|up|down' and
+    'l<i>.mlp.shared.gate|up|down' (mixture).  Linear weights are [out, in]."""
+    spec, W = cfg.hybrid, cfg.hidden_size
+
+    def put(t, dt=dtype):
+        return t.to(dt).contiguous().to(device)
+
+    def f32(t):
+        return put(t.reshape(-1), torch.float32)
+
+    def expect(name, shape):
+        t = get(name)
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"{name}: shape {tuple(t.shape)}, expected {tuple(shape)}")
+        return t
+
+    w = ModelWeights(embed=put(expect("embed", (cfg.vocab_size, W))))
+    pos = get("pos")
+    if pos.dim() != 2 or pos.shape[1] != W:
+        raise ValueError(f"pos: shape {tuple(pos.shape)}, expected [positions, {W}]")
+    w.pos_embed = put(pos)
+    for i, L in enumerate(spec.layers):
+        p, m, q = f"l{i}.", f"l{i}.mix.", f"l{i}.mlp."
+        A = L.battn
+        parts = [("q", expect(m + "q", (A.heads * A.dim, W)))]
+        if A.kv_from is None:
+            parts += [("k", expect(m + "k", (A.kv_heads * A.dim, W))), ("v", expect(m + "v", (A.kv_heads * A.vdim, W)))]
+        parts.append(("g", expect(m + "g", (A.heads, W))))
+        outs = [expect(m + "o", (W, A.heads * A.vdim))]
+        ff = L.ff if L.ff else (L.moe.shared_ff if L.moe is not None else 0)
+        if ff:
+            r = q if L.ff else q + "shared."
+            parts += [("gate", expect(r + "gate", (ff, W))), ("up", expect(r + "up", (ff, W)))]
+            outs.append(expect(r + "down", (W, ff)))
+        in_w, seg = _fuse_segments(parts, W, put)
+        in_b = None
+        if A.bias:
+            b = torch.zeros(in_w.shape[0], dtype=torch.float32)
+            for n, _ in parts[: 3 if A.kv_from is None else 1]:
+                b[seg[n][0]: seg[n][0] + seg[n][1]] = expect(m + n + ".b", (seg[n][1],)).float()
+            in_b = put(b)
+        # the row that out_w multiplies: the heads, then the activated hidden units on a 16-byte boundary
+        n_attn = -(-A.heads * A.vdim // 8) * 8
+        out_w = torch.zeros(W, n_attn + ff, dtype=outs[0].dtype)
+        out_w[:, : A.heads * A.vdim] = outs[0]
+        if ff:
+            out_w[:, n_attn:] = outs[1]
+        lw = ParallelLayerWeights(norm1=put(expect(p + "norm1", (W,))), in_w=in_w, in_b=in_b, seg=seg, out_w=put(out_w),
+                                  sink=torch.full((A.heads,), float(A.sink), dtype=torch.float32, device=device)
+                                  if A.sink is not None else None)
+        if L.moe is not None:
+            M = L.moe
+            lw.router_w = put(expect(q + "router", (M.experts, W)), torch.float32)
+            lw.router_b = f32(expect(q + "router.b", (M.experts,))) if M.router_bias else None
+            lw.correction = torch.zeros(M.experts, dtype=torch.float32, device=device)
+            lw.gate_up_w = put(torch.stack([torch.cat([expect(f"{q}e{e}.gate", (M.ff, W)), expect(f"{q}e{e}.up", (M.ff, W))],
+                                                      dim=0) for e in range(M.experts)]))
+            lw.down_w = put(torch.stack([expect(f"{q}e{e}.down", (W, M.ff)) for e in range(M.experts)]))
+        w.layers.append(lw)
+    w.final_norm = put(expect("final.norm", (W,)))
+    w.lm_head = put(expect("head", (cfg.vocab_size, W)))
+    return w
+
+
+def bemulorn_synthetic_state(cfg: ModelConfig, seed: int = 0, device="cpu", dtype=torch.float32) -> dict:
+    """Seeded random tensors under a Bemulorn checkpoint's names (benchmarks and tests: nothing can be
+    downloaded)."""
+    spec, W = cfg.hybrid, cfg.hidden_size
+    gen = torch.Generator(device=device).manual_seed(seed)
+
+    def mat(*shape, s=1.0):
+        return torch.empty(shape, dtype=dtype, device=device).normal_(0.0, s, generator=gen)
+
+    def near(value, *shape, s=0.1):
+        return torch.full(shape, float(value), dtype=dtype, device=device) + mat(*shape, s=s)
+
+    st = {"embed": mat(cfg.vocab_size, W), "pos": mat(cfg.max_position_embeddings, W, s=0.5),
+          "head": mat(cfg.vocab_size, W, s=W ** -0.5), "final.norm": near(1.0, W)}
+    for i, L in enumerate(spec.layers):
+        p, m, q = f"l{i}.", f"l{i}.mix.", f"l{i}.mlp."
+        A = L.battn
+        st[p + "norm1"] = near(1.0, W)
+        st[m + "q"], st[m + "q.b"] = mat(A.heads * A.dim, W, s=W ** -0.5), mat(A.heads * A.dim, s=0.2)
+        if A.kv_from is None:
+            st[m + "k"], st[m + "k.b"] = mat(A.kv_heads * A.dim, W, s=W ** -0.5), mat(A.kv_heads * A.dim, s=0.2)
+            st[m + "v"], st[m + "v.b"] = mat(A.kv_heads * A.vdim, W, s=W ** -0.5), mat(A.kv_heads * A.vdim, s=0.2)
+        st[m + "g"] = mat(A.heads, W, s=W ** -0.5)
+        st[m + "o"] = mat(W, A.heads * A.vdim, s=(A.heads * A.vdim) ** -0.5)
+        if L.ff:
+            st[q + "gate"], st[q + "up"] = mat(L.ff, W, s=W ** -0.5), mat(L.ff, W, s=W ** -0.5)
+            st[q + "down"] = mat(W, L.ff, s=L.ff ** -0.5)
+        elif L.moe is not None:
+            M = L.moe
+            st[q + "router"], st[q + "router.b"] = mat(M.experts, W, s=W ** -0.5), mat(M.experts, s=0.3)
+            for e in range(M.experts):
+                st[f"{q}e{e}.gate"], st[f"{q}e{e}.up"] = mat(M.ff, W, s=W ** -0.5), mat(M.ff, W, s=W ** -0.5)
+                st[f"{q}e{e}.down"] = mat(W, M.ff, s=M.ff ** -0.5)
+            if M.shared_ff:
+                st[q + "shared.gate"], st[q + "shared.up"] = mat(M.shared_ff, W, s=W ** -0.5), mat(M.shared_ff, W, s=W ** -0.5)
+                st[q + "shared.down"] = mat(W, M.shared_ff, s=M.shared_ff ** -0.5)
+    return st
+
+
 def tafisun_synthetic_state(cfg: ModelConfig, seed: int = 0, device="cpu", dtype=torch.float32) -> dict:
     """Seeded random tensors under a Tafisun checkpoint's names (benchmarks and tests: nothing can be
     downloaded)."""
@@ -674,6 +812,8 @@ def hybrid_synthetic_state(cfg: ModelConfig, seed: int = 0, std: float = 0.02, r
         return sandwich_synthetic_state(cfg, seed=seed, device=device, dtype=dtype)
     if cfg.architecture == "Tafisun":
         return tafisun_synthetic_state(cfg, seed=seed, device=device, dtype=dtype)
+    if spec.arrangement == "parallel":
+        return bemulorn_synthetic_state(cfg, seed=seed, device=device, dtype=dtype)
     gen = torch.Generator(device=device).manual_seed(seed)
 
     def mat(*shape, s=std):

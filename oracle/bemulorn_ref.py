@@ -108,43 +108,60 @@ def keys_values(wt, pre, m, h, dtype=torch.float32):
     return k, v
 
 
+def attend(q, k, v, scale, size, gate_logits=None, sink=True):
+    """q [T, H, d] and k [T, G, d] as they enter the scores (rotated already), v [T, G, dv], all of one
+    sequence from position 0; gate_logits [T, H] or None.  Returns [T, H * dv]."""
+    T, H = q.shape[0], q.shape[1]
+    rep = H // k.shape[1]
+    ke, ve = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)      # query head h uses head h // rep
+    s = torch.einsum("ihd,jhd->hij", q, ke) * scale
+    ok = chunk_mask(T, size)
+    p = sink_softmax(s, ok) if sink else torch.softmax(s.masked_fill(~ok, float("-inf")), dim=-1)
+    o = torch.einsum("hij,jhc->ihc", p, ve)
+    if gate_logits is not None:
+        o = o * torch.sigmoid(gate_logits)[:, :, None]
+    return o.reshape(T, -1)
+
+
 def attention(wt, pre, m, h, kv, dtype=torch.float32):
     """h [T, W] (a whole sequence from position 0), kv = (keys, values) of this layer or of the
     layer it shares with.  Returns the mixer's output [T, W]."""
     T = h.shape[0]
-    H, G, d, dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+    H, d = int(m["heads"]), int(m["dim"])
     q = (h @ wt[pre + "q"].to(dtype).T + wt[pre + "q.b"].to(dtype)).view(T, H, d)
     rot = m.get("rot")
     if rot and int(rot["dims"]) > 0:
         cos, sin = rotary_angles(rot, T, dtype)
         q = rotate(q, cos, sin, int(rot["dims"]))
-    k, v = kv
-    rep = H // G
-    ke, ve = k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1)      # query head h uses head h // rep
-    s = torch.einsum("ihd,jhd->hij", q, ke) * float(m["scale"])
-    p = sink_softmax(s, chunk_mask(T, int((m.get("mask") or {}).get("size") or 0)))
-    o = torch.einsum("hij,jhc->ihc", p, ve)
-    gate = torch.sigmoid(h @ wt[pre + "g"].to(dtype).T)                           # [T, H]
-    return (o * gate[:, :, None]).reshape(T, H * dv) @ wt[pre + "o"].to(dtype).T
+    o = attend(q, kv[0], kv[1], float(m["scale"]), int((m.get("mask") or {}).get("size") or 0), h @ wt[pre + "g"].to(dtype).T)
+    return o @ wt[pre + "o"].to(dtype).T
+
+
+def limited_unit(g, u, limit):
+    g, u = torch.clamp(g, max=limit), torch.clamp(u, min=-limit, max=limit)
+    return g * torch.sigmoid(1.702 * g) * (u + 1.0)
+
+
+def silu_unit(g, u):
+    return g * torch.sigmoid(g) * u
 
 
 def limited_ff(wt, pre, h, limit, dtype=torch.float32):
-    g = torch.clamp(h @ wt[pre + "gate"].to(dtype).T, max=limit)
-    u = torch.clamp(h @ wt[pre + "up"].to(dtype).T, min=-limit, max=limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ wt[pre + "down"].to(dtype).T
+    return limited_unit(h @ wt[pre + "gate"].to(dtype).T, h @ wt[pre + "up"].to(dtype).T, limit) @ wt[pre + "down"].to(dtype).T
 
 
 def silu_ff(wt, pre, h, dtype=torch.float32):
-    g = h @ wt[pre + "gate"].to(dtype).T
-    return (g * torch.sigmoid(g) * (h @ wt[pre + "up"].to(dtype).T)) @ wt[pre + "down"].to(dtype).T
+    return silu_unit(h @ wt[pre + "gate"].to(dtype).T, h @ wt[pre + "up"].to(dtype).T) @ wt[pre + "down"].to(dtype).T
+
+
+def choose(z, top):
+    """z float32 [T, experts] -> (ids [T, top], weights [T, top]): the largest logits, a softmax over them alone."""
+    val, ids = torch.topk(z, top, dim=-1)
+    return ids, torch.softmax(val, dim=-1)
 
 
 def route(wt, pre, mlp, h):
-    """(ids [T, top], weights [T, top]) in float32."""
-    z = h.float() @ wt[pre + "router"].float().T + wt[pre + "router.b"].float()
-    top = int(mlp["router"]["top"])
-    val, ids = torch.topk(z, top, dim=-1)
-    return ids, torch.softmax(val, dim=-1)
+    return choose(h.float() @ wt[pre + "router"].float().T + wt[pre + "router.b"].float(), int(mlp["router"]["top"]))
 
 
 def mixture(wt, pre, mlp, h, dtype=torch.float32):
@@ -185,3 +202,44 @@ def forward(wt, cfg, tokens, dtype=torch.float32, layers_out=None):
             layers_out.append(x.clone())
     h = rms_norm(x, wt["final.norm"].to(dtype), eps)
     return h @ wt["head"].to(dtype).T * float(cfg.get("logit_scale", 1.0))
+
+
+def random_state(cfg, seed=0, bf16_grid=True):
+    """Seeded random tensors under the checkpoint names of `cfg` (a config dict), float32; with
+    bf16_grid every value is representable in bfloat16."""
+    g = torch.Generator().manual_seed(seed)
+    W, V = cfg["width"], cfg["vocab"]
+
+    def mat(*shape, s=1.0, mean=0.0):
+        t = torch.randn(tuple(shape), generator=g) * s + mean
+        return t.to(torch.bfloat16).float() if bf16_grid else t
+
+    st = {"embed": mat(V, W), "pos": mat(cfg["max_positions"], W, s=0.7), "head": mat(V, W, s=W ** -0.5),
+          "final.norm": mat(W, s=0.1, mean=1.0)}
+    for i, L in enumerate(cfg["layers"]):
+        p, q, f = f"l{i}.", f"l{i}.mix.", f"l{i}.mlp."
+        m = L["mixer"]
+        H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        st[p + "norm1"] = mat(W, s=0.1, mean=1.0)
+        st[q + "q"], st[q + "q.b"] = mat(H * d, W, s=W ** -0.5), mat(H * d, s=0.3)
+        if m.get("kv_from") is None:
+            st[q + "k"], st[q + "k.b"] = mat(G * d, W, s=W ** -0.5), mat(G * d, s=0.3)
+            st[q + "v"], st[q + "v.b"] = mat(G * dv, W, s=W ** -0.5), mat(G * dv, s=0.3)
+        st[q + "g"], st[q + "o"] = mat(H, W, s=W ** -0.5), mat(W, H * dv, s=(H * dv) ** -0.5)
+        mlp = L.get("mlp")
+        if mlp is None:
+            continue
+        if mlp.get("kind", "dense") == "dense":
+            F = mlp["ff"]
+            st[f + "gate"], st[f + "up"], st[f + "down"] = mat(F, W, s=W ** -0.5), mat(F, W, s=W ** -0.5), mat(W, F, s=F ** -0.5)
+            continue
+        r, F = mlp["router"], mlp["expert"]["ff"]
+        st[f + "router"], st[f + "router.b"] = mat(r["experts"], W, s=2.0 * W ** -0.5), mat(r["experts"], s=0.5)
+        for e in range(r["experts"]):
+            st[f"{f}e{e}.gate"], st[f"{f}e{e}.up"] = mat(F, W, s=W ** -0.5), mat(F, W, s=W ** -0.5)
+            st[f"{f}e{e}.down"] = mat(W, F, s=F ** -0.5)
+        if mlp.get("shared"):
+            S = mlp["shared"]["ff"]
+            st[f + "shared.gate"], st[f + "shared.up"] = mat(S, W, s=W ** -0.5), mat(S, W, s=W ** -0.5)
+            st[f + "shared.down"] = mat(W, S, s=S ** -0.5)
+    return st

@@ -142,10 +142,10 @@ def parse():
                     help="instead of the default workload: prefill and decode throughput of hybrid (Lozupel) decoders at a "
                          "few real layer sizes beside Llama-shaped decoders of equal size, and the hybrid kernels' times "
                          "against their rooflines beside the like kernels of the Llama path (random weights)")
-    ap.add_argument("--hybrid-design", default="lozupel", choices=("lozupel", "tativik", "tafisun"),
-                    help="with --hybrid-compare: lozupel (beside Llama-shaped decoders), tativik (beside Lozupel decoders) or "
-                         "tafisun (beside Tativik decoders) "
-                         "of equal width and depth, the closest existing model)")
+    ap.add_argument("--hybrid-design", default="lozupel", choices=("lozupel", "tativik", "tafisun", "bemulorn"),
+                    help="with --hybrid-compare: lozupel (beside Llama-shaped decoders), tativik (beside Lozupel decoders), "
+                         "tafisun (beside Tativik decoders) or bemulorn (beside Llama-shaped decoders) "
+                         "of equal width and depth, the closest existing model")
     ap.add_argument("--hybrid-widths", default="2048,4096")
     ap.add_argument("--hybrid-layers", type=int, default=4)
     return ap.parse_args()
@@ -610,8 +610,8 @@ def pmc_traffic(tiled):
 def main():
     a = parse()
     if a.hybrid_compare:
-        from mi355_decode.bench_hybrid import compare, compare_tafisun, compare_tativik
-        print(json.dumps({"tativik": compare_tativik, "tafisun": compare_tafisun}.get(a.hybrid_design, compare)([int(w) for w in a.hybrid_widths.split(",")], a.hybrid_layers, a.batch_per_gpu,
+        from mi355_decode.bench_hybrid import compare, compare_bemulorn, compare_tafisun, compare_tativik
+        print(json.dumps({"tativik": compare_tativik, "tafisun": compare_tafisun, "bemulorn": compare_bemulorn}.get(a.hybrid_design, compare)([int(w) for w in a.hybrid_widths.split(",")], a.hybrid_layers, a.batch_per_gpu,
                                  a.prompt_len if a.prompt_len != 128 else 2048, min(a.steps, 64), a.warmup)), flush=True)
         return
     if a.gpus > 1 and "WORLD_SIZE" not in os.environ:

@@ -238,6 +238,61 @@ def block_mixer_generation():
     return out
 
 
+def parallel_layer_generation():
+    """A hybrid decoder of the Bemulorn design (one norm per layer, attention in chunks with rotary
+    positions, a value-less softmax term and shared pages, a limited gated unit and a mixture with a
+    shared expert): the same schedule as above, in bfloat16 and in float32."""
+    from mi355_decode import weights as W
+    from mi355_decode.config import EngineArgs, ModelConfig
+    from mi355_decode.llm import build_engine
+    from mi355_decode.sampling_params import SamplingParams
+    rot = {"dims": 16, "base": 10000.0, "scaling": {"factor": 2.0, "original": 64, "fast": 16.0, "slow": 1.0}}
+    att = {"heads": 8, "kv_heads": 2, "dim": 32, "vdim": 16, "mask": {"size": 40}, "scale": 0.2, "rot": rot}
+    moe = {"kind": "moe", "expert": {"ff": 64}, "shared": {"ff": 48}, "router": {"experts": 6, "top": 2}}
+    cfg = ModelConfig.from_dict({
+        "architecture": "Bemulorn", "width": 128, "vocab": 300, "max_positions": 256, "norm": {"eps": 1e-6},
+        "embedding": {"scale": 2.0}, "logit_scale": 0.5,
+        "layers": [{"type": "attention", "mixer": att, "mlp": {"kind": "dense", "ff": 192, "limit": 2.0}},
+                   {"type": "attention", "mixer": dict(att, heads=4, kv_from=0, mask={"size": 7}), "mlp": moe},
+                   {"type": "attention", "mixer": dict(att, heads=3, kv_heads=1, dim=40, vdim=9, mask=None), "mlp": None},
+                   {"type": "attention", "mixer": dict(att, heads=2, kv_from=0), "mlp": dict(moe, shared=None)}]})
+    state = W.hybrid_synthetic_state(cfg, seed=3)
+    rng = np.random.default_rng(1)
+    out = []
+    for dtype in ("bfloat16", "float32"):
+        bounds.clear()
+        eng = build_engine(EngineArgs(model="chunks", dtype=dtype, max_num_seqs=4, max_model_len=256,
+                                      num_gpu_blocks_override=48, gpu_memory_utilization=0.0, max_num_batched_tokens=1 << 20),
+                           state_dict=state, model_config=cfg)
+
+        def run(tag):
+            toks = {r: rng.integers(0, 300, n).tolist() for r, n in (("a", 150), ("b", 37), ("c", 2))}
+            eng.forced_step([(tag + "a", toks["a"][:100], [99]), (tag + "c", toks["c"][:1], [0])])
+            eng.forced_step([(tag + "a", toks["a"][100:102], [1]), (tag + "b", toks["b"][:33], []), (tag + "c", toks["c"][1:], [0])],
+                            [tag + "c"])
+            for i in range(4):
+                eng.forced_step([(tag + "a", toks["a"][102 + i:103 + i], [0]), (tag + "b", toks["b"][33 + i:34 + i], [0])])
+            eng.forced_step([(tag + "a", toks["a"][106:], [])], [tag + "a", tag + "b"])
+            for i, n in enumerate((5, 70, 17)):
+                eng.add_request(f"{tag}g{i}", rng.integers(0, 300, n).tolist(),
+                                SamplingParams(max_tokens=10, temperature=0.0 if i else 0.8, seed=i, ignore_eos=True))
+            n = 0
+            while eng.has_unfinished():
+                n += sum(len(o.new_token_ids) for o in eng.step())
+            return n
+
+        run("warm")
+        n = bounds.sync_allocations(granularity="segment")
+        toks = run("checked")
+        rep = bounds.report()
+        assert rep is None or rep["refused"] == 0, (dtype, rep)
+        out.append(f"{dtype}:{toks} tokens:{n} segments:{rep['unknown_base'] if rep else 0} accesses with an unlisted base")
+        del eng
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
 def sampler_rows():
     """The sampling launch on exactly sized logits (no slack behind the last row), every kind of
     row in one call: greedy, whole-vocabulary draw, top-k / top-p cuts, an all-tied row (the list
@@ -277,4 +332,5 @@ if __name__ == "__main__":
     res["engine"] = engine_generation()
     res["sandwich"] = sandwich_generation()
     res["block_mixers"] = block_mixer_generation()
+    res["parallel_layers"] = parallel_layer_generation()
     print(json.dumps(res))

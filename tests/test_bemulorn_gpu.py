@@ -360,10 +360,11 @@ def test_routing_by_logits_with_a_softmax_over_the_chosen(E, top):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("limit", [None, 0.4, 7.0])
-def test_gated_activation_on_column_slices(dtype, limit):
+@pytest.mark.parametrize("F", [27, 32])                     # (32: eight hidden units per thread in 16 bits)
+def test_gated_activation_on_column_slices(dtype, limit, F):
     from mi355_decode import ops
     g = torch.Generator().manual_seed(5)
-    T, F = 19, 27
+    T = 19
     buf = (torch.randn(T, 8 + 2 * 32, generator=g) * 3).to(dtype)
     gate, up = buf[:, 8: 8 + F], buf[:, 40: 40 + F]
     row = torch.full((T, 40), float("nan"), dtype=dtype, device="cuda")

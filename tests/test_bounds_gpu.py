@@ -34,4 +34,4 @@ def test_no_access_leaves_its_allocation():
     print(json.dumps(res, indent=1))
     assert res["negative_control"]["refused"] > 0
     assert len(res["rank_steps"]) == 18 and len(res["engine"]) == 3 and len(res["sampler"]) == 12
-    assert len(res["sandwich"]) == 2 and len(res["block_mixers"]) == 2
+    assert len(res["sandwich"]) == 2 and len(res["block_mixers"]) == 2 and len(res["parallel_layers"]) == 2

@@ -162,7 +162,9 @@ __global__ __launch_bounds__(64) void softmax_bias_attn_kernel(
 // lie in two blocks: the walk starts at the first row's block and every row masks for itself.
 // gridDim.z > 1: the 32-key tiles are dealt out to the z workgroups in turn, each leaves its
 // accumulators, maxima and sums in fp32 scratch, and bias_attn_merge_kernel joins them.
-template <typename T, int HB, int DS, int CB>
+// DS / CB: fragment counts the registers are sized for (2 / 4 for heads of up to 64 channels, else
+// 4 / 8); PEN: the distance penalty is computed (off: no logarithm per score).
+template <typename T, int HB, int DS, int CB, bool PEN>
 __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
     uint16_t* __restrict__ out, const uint16_t* __restrict__ q, int64_t q_stride, const uint16_t* __restrict__ k_cache,
     const uint16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
@@ -171,10 +173,21 @@ __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
     int d, int dv, int block, int window, float scale, float* __restrict__ part_acc, float* __restrict__ part_ml,
     int64_t total_rows, const float* __restrict__ sink, int64_t out_stride) {
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int tile = blockIdx.x * (blockDim.x >> 6) + wave;
+  // Workgroups go to the 8 XCDs in turn (x fastest), each XCD with an L2 of its own.  Where the plane of
+  // workgroups divides by 8, XCD k takes the k-th eighth of the (head group, tile) pairs in head-major order:
+  // the tiles of one kv head then read its K/V through one L2 instead of through all eight.
+  int bx = blockIdx.x, by = blockIdx.y;
+  const int plane = gridDim.x * gridDim.y;
+  if (plane % 8 == 0) {
+    const int lin = blockIdx.x + blockIdx.y * gridDim.x;
+    const int v = (lin & 7) * (plane >> 3) + (lin >> 3);
+    bx = v % gridDim.x;
+    by = v / gridDim.x;
+  }
+  const int tile = bx * (blockDim.x >> 6) + wave;
   if (tile >= num_tiles) return;                        // (no workgroup barrier below)
   const int rep = H / G, hbs = rep / HB;
-  const int g = blockIdx.y / hbs, h0 = g * rep + (blockIdx.y % hbs) * HB;
+  const int g = by / hbs, h0 = g * rep + (by % hbs) * HB;
   const int nz = gridDim.z, z = blockIdx.z;
   const int li = lane & 15, kk = lane >> 4;
   const int seq = MI355_LD(int32_t, tiles, tiles + 3 * tile);
@@ -200,8 +213,8 @@ __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
       if (s < ds && valid)
         qf[i][s] = MI355_LD(uint4, q, q + (row0 + li) * q_stride + static_cast<int64_t>(h0 + i) * d + 32 * s + 8 * kk);
     }
-    a1[i] = r1 != nullptr ? MI355_LD(float, r1, r1 + h0 + i) : 0.f;      // ln(x) r1 = log2(x) r1 ln 2, times log2 e again: r1
-    a2[i] = r2 != nullptr ? MI355_LD(float, r2, r2 + h0 + i) : 0.f;
+    a1[i] = PEN ? MI355_LD(float, r1, r1 + h0 + i) : 0.f;               // ln(x) r1 = log2(x) r1 ln 2, times log2 e again: r1
+    a2[i] = PEN ? MI355_LD(float, r2, r2 + h0 + i) : 0.f;
     m[i] = -1.0e30f;
     l[i] = 0.f;
 #pragma unroll
@@ -259,7 +272,7 @@ __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
       for (int r = 0; r < 4; ++r) {
         const int64_t key = base + 16 * half + 4 * kk + r;
         vis[half][r] = valid && key <= my_p && key >= my_lo;
-        dist[half][r] = vis[half][r] ? static_cast<float>(my_p - key) : 0.f;
+        dist[half][r] = PEN && vis[half][r] ? static_cast<float>(my_p - key) : 0.f;
       }
     }
     uint32_t pw[HB][4];
@@ -278,7 +291,8 @@ __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           // base 2 throughout: q.k scale log2(e) - r1 log2(1 + r2 dist)
-          sc[half][r] = sacc[r] * scale2 - a1[i] * __builtin_amdgcn_logf(1.0f + a2[i] * dist[half][r]);
+          sc[half][r] = sacc[r] * scale2;
+          if (PEN) sc[half][r] -= a1[i] * __builtin_amdgcn_logf(1.0f + a2[i] * dist[half][r]);
           if (vis[half][r]) tmax = fmaxf(tmax, sc[half][r]);
         }
       }
@@ -508,6 +522,7 @@ extern "C" int32_t mi355_softmax_bias_attn(void* out, const void* q, int64_t q_s
     const bool split = workspace != nullptr && num_splits > 1;
     MI355_REQUIRE(num_splits >= 0 && num_splits <= 64, MI355_ERR_INVALID, "softmax_bias_attn: %d key splits", num_splits);
     const int hb = rep % 4 == 0 ? 4 : rep % 3 == 0 ? 3 : rep % 2 == 0 ? 2 : 1;
+    const bool small = head_dim <= 64 && v_dim <= 64;       // half the fragments: registers for a second wave per SIMD
     const int waves = num_tiles < 4 ? num_tiles : 4;                              // a tile per wave
     const dim3 grid(static_cast<unsigned>((num_tiles + waves - 1) / waves), static_cast<unsigned>(num_kv_heads * (rep / hb)),
                     split ? num_splits : 1);
@@ -516,7 +531,14 @@ extern "C" int32_t mi355_softmax_bias_attn(void* out, const void* q, int64_t q_s
     float* part_acc = split ? workspace : nullptr;
     float* part_ml = split ? workspace + static_cast<int64_t>(num_splits) * pairs * v_dim : nullptr;
 #define MI355_BMFMA(TT, HB)                                                                                         \
-  hipLaunchKernelGGL((softmax_bias_attn_mfma_kernel<TT, HB, 4, 8>), grid, block_dim, 0, s,                          \
+  do {                                                                                                              \
+    if (small && r1 != nullptr) MI355_BMFMA_K(TT, HB, 2, 4, true);                                                  \
+    else if (small) MI355_BMFMA_K(TT, HB, 2, 4, false);                                                             \
+    else if (r1 != nullptr) MI355_BMFMA_K(TT, HB, 4, 8, true);                                                      \
+    else MI355_BMFMA_K(TT, HB, 4, 8, false);                                                                        \
+  } while (0)
+#define MI355_BMFMA_K(TT, HB, DS, CB, PEN)                                                                          \
+  hipLaunchKernelGGL((softmax_bias_attn_mfma_kernel<TT, HB, DS, CB, PEN>), grid, block_dim, 0, s,                   \
                      static_cast<uint16_t*>(out), static_cast<const uint16_t*>(q), q_stride,                        \
                      static_cast<const uint16_t*>(k_cache), static_cast<const uint16_t*>(v_cache), block_tables,    \
                      max_blocks, tiles, num_tiles, positions, r1, r2, static_cast<const uint16_t*>(gate),           \
@@ -539,6 +561,7 @@ extern "C" int32_t mi355_softmax_bias_attn(void* out, const void* q, int64_t q_s
   } while (0)
     if (dtype == MI355_BF16) MI355_BMFMA_HB(BF16); else MI355_BMFMA_HB(F16);
 #undef MI355_BMFMA_HB
+#undef MI355_BMFMA_K
 #undef MI355_BMFMA
     return check_launch("softmax_bias_attn (matrix cores)");
   }

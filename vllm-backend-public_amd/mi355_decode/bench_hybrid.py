@@ -59,6 +59,23 @@ def tafisun_config(width: int, layers: int, vocab: int = 32000) -> dict:
             "embedding": {"bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 7919}}, "layers": ls}
 
 
+def bemulorn_config(width: int, layers: int, vocab: int = 32000, max_positions: int = 4096) -> dict:
+    """Attention layers with parallel sub-layers: 128-wide heads, four query heads to a key head,
+    chunks of 1024 positions, rotary positions on half of every head with blended frequencies; the
+    second half of the layers reads the pages of the last layer of the first half; a limited gated
+    feed-forward of 2 * width in the even layers and, in the odd ones, 32 experts of width / 2 with 4 per
+    token beside a shared expert of width / 2."""
+    nh = width // 128
+    rot = {"dims": 64, "base": 10000.0, "scaling": {"factor": 4.0, "original": 1024, "fast": 32.0, "slow": 1.0}}
+    att = {"heads": nh, "kv_heads": max(nh // 4, 1), "dim": 128, "vdim": 128, "mask": {"size": 1024}, "scale": 128 ** -0.5, "rot": rot}
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "shared": {"ff": width // 2}, "router": {"experts": 32, "top": 4}}
+    own = max(layers // 2, 1)
+    ls = [{"type": "attention", "mixer": att if i < own else dict(att, kv_from=own - 1),
+           "mlp": {"kind": "dense", "ff": 2 * width, "limit": 7.0} if i % 2 == 0 else moe} for i in range(layers)]
+    return {"architecture": "Bemulorn", "width": width, "vocab": vocab, "max_positions": max_positions, "norm": {"eps": 1e-6},
+            "embedding": {"scale": 2.0}, "logit_scale": 0.5, "layers": ls}
+
+
 def lozupel_config(width: int, layers: int, vocab: int = 32000, loop: bool = True) -> dict:
     """Alternating parallel / delta layers with 128-wide heads, a 1024-token window, a feed-forward in
     every layer; the middle of the stack loops twice."""
@@ -563,4 +580,144 @@ def compare_tafisun(widths, layers: int, batch: int, prompt_len: int, steps: int
                                  "prefill_ratio": round(t["prefill_tok_s"] / z["prefill_tok_s"], 3),
                                  "decode_ratio": round(t["decode_tok_s"] / z["decode_tok_s"], 3)})
         result["kernels"][str(width)] = tafisun_kernel_table(width, prompt_len, batch)
+    return result
+
+
+def bemulorn_kernel_table(width: int, prompt_len: int, batch: int) -> list:
+    """The Bemulorn design's kernels at the prefill and the decode shape, each against its own
+    roofline, beside the like kernel of the closest existing paths (the Llama-shaped decoder's for
+    attention, norm and activation; the Tafisun design's mixture) at the same shape."""
+    from types import SimpleNamespace
+    from .config import MoESpec, RotaryScaling
+    from .hybrid_runner import MoEFeedForward, rotary_table
+    dev, bf = "cuda", torch.bfloat16
+    g = torch.Generator(device=dev).manual_seed(0)
+    rnd = lambda *s, dt=bf: torch.randn(*s, device=dev, dtype=torch.float32, generator=g).to(dt)  # noqa: E731
+    rows = []
+
+    def row(kernel, shape, t, bound, work, like=None, like_t=None, like_work=None, like_bound=None):
+        peak = {"hbm": HBM, "mfma": MFMA, "valu": VALU}
+        r = {"kernel": kernel, "shape": shape, "us": round(t * 1e6, 2), "bound": bound,
+             "frac_of_roofline": round(work / peak[bound] / t, 4)}
+        if like is not None:
+            r.update(like=like, like_us=round(like_t * 1e6, 2), like_frac=round(like_work / peak[like_bound or bound] / like_t, 4))
+            r["distance_ratio"] = round(r["like_frac"] / max(r["frac_of_roofline"], 1e-9), 2)
+        rows.append(r)
+
+    P, W, V = prompt_len, width, 32000
+    H, G, d, chunk = W // 128, max(W // 512, 1), 128, 1024
+    pages = (P + BLOCK_SIZE) // BLOCK_SIZE + 1
+    nb = pages * batch
+    kc, vct = rnd(nb, G, BLOCK_SIZE, d), rnd(nb, G, d, BLOCK_SIZE)
+    bt = torch.arange(nb, dtype=torch.int32, device=dev).view(batch, pages)
+    embed, ptab = rnd(V, W), rnd(pages * BLOCK_SIZE, W)
+    sink = torch.zeros(H, device=dev)
+    cs = rotary_table(64, 10000.0, pages * BLOCK_SIZE, dev, RotaryScaling(4.0, 1024.0, 32.0, 1.0))
+    F = 2 * W
+    for T, S, tag in ((P, 1, "prefill"), (batch, batch, "decode")):
+        shape = f"{tag} {T} rows x {W}"
+        per = T // S
+        pos = (torch.arange(T, device=dev) % per + (0 if S == 1 else P - 1)).to(torch.int64)
+        seq = (torch.arange(T, device=dev) // per).to(torch.int32)
+        ids = torch.randint(0, V, (T,), device=dev, generator=g)
+        # ---- embedding
+        row("embed_scale_pos_f32", shape, _time(lambda: ops.embed_scale_pos_f32(embed, ids, 2.0, ptab, pos)), "hbm", T * W * 8,
+            "embed_scale_f32", _time(lambda: ops.embed_scale_f32(embed, ids, 2.0)), T * W * 6)
+        # ---- the one norm of a layer, the previous layer's output riding in its launch
+        resid, add16, wv = rnd(T, W, dt=torch.float32), rnd(T, W), rnd(W)
+        x16, r16, out16 = rnd(T, W), rnd(T, W), torch.empty(T, W, device=dev, dtype=bf)
+        row("add_rms_norm_f32 (vector weight)", shape, _time(lambda: ops.add_rms_norm_f32(resid, wv, 1e-6, add=add16, out=out16)),
+            "hbm", T * W * 12, "fused_add_rms_norm", _time(lambda: ops.fused_add_rms_norm(x16, r16, wv, 1e-6, out=out16)), T * W * 8)
+        # ---- the gated activation: column slices of the fused projection into a slice of the output row
+        proj = rnd(T, (H + 2 * G) * d + 8 + 2 * F)
+        at = (H + 2 * G) * d + 8
+        rowbuf = torch.empty(T, H * d + F, device=dev, dtype=bf)
+        gu, act = rnd(T, 2 * F), torch.empty(T, F, device=dev, dtype=bf)
+        row("gated_act_rows (limited unit, column slices)", f"{tag} {T} rows x {F}",
+            _time(lambda: ops.gated_act_rows(proj[:, at: at + F], proj[:, at + F: at + 2 * F], 7.0, out=rowbuf[:, H * d:])), "hbm",
+            T * F * 6, "silu_and_mul", _time(lambda: ops.silu_and_mul(gu, out=act)), T * F * 6)
+        # ---- rotation and page write
+        q, k, v_ = proj[:, : H * d], proj[:, H * d: (H + G) * d], proj[:, (H + G) * d: (H + 2 * G) * d]
+        gh = proj[:, (H + 2 * G) * d: (H + 2 * G) * d + H]
+        wslots = (torch.arange(T, device=dev) if S == 1 else torch.arange(T, device=dev) * pages * BLOCK_SIZE + P - 1).to(torch.int64)
+        wn = torch.ones(d, device=dev)
+        row("rope_partial_kv_write (64 of 128 rotated)", f"{tag} {T} rows, {H}/{G} heads x {d}",
+            _time(lambda: ops.rope_partial_kv_write(q, k, v_, cs, pos, wslots, kc, vct, H, G, d, d)), "hbm",
+            T * (2 * H * d + 4 * G * d) * 2,
+            "qk_norm_kv_write", _time(lambda: ops.qk_norm_kv_write(q, k, k, wn, wn, wslots, kc, vct, H, G, d, d, 1e-6)),
+            T * (2 * H * d + 3 * G * d) * 2)
+        row("rope_partial_kv_write (queries alone: shared pages)", f"{tag} {T} rows, {H} heads x {d}",
+            _time(lambda: ops.rope_partial_kv_write(q, None, None, cs, pos, wslots, None, None, H, G, d, d)), "hbm",
+            T * 2 * H * d * 2)
+        # ---- attention beside the Llama path's
+        if S == 1:
+            tiles = torch.from_numpy(ops.query_tiles([0, P])).to(dev)
+            b_t = bt[:1]
+        else:
+            tiles = torch.stack([seq, seq, torch.ones_like(seq)], dim=1).contiguous()
+            b_t = bt
+        rep = H // G
+        hb = 4 if rep % 4 == 0 else 3 if rep % 3 == 0 else 2 if rep % 2 == 0 else 1
+        nsb = max(min(16, chunk // 64, 1024 // max(int(tiles.shape[0]) * G * (rep // hb), 1)), 1)
+        out_slice = rowbuf[:, : H * d]
+        t_n = _time(lambda: ops.softmax_bias_attn(q, kc, vct, b_t, seq, pos, None, None, gh, H, d ** -0.5, block=chunk, tiles=tiles,
+                                                  num_splits=nsb if nsb > 1 else 0, sink=sink, out=out_slice), 5)
+        o = torch.empty(T, H * d, device=dev, dtype=bf)
+        qc = q.contiguous()
+        if S == 1:
+            cu, ctx = torch.tensor([0, P], dtype=torch.int32, device=dev), torch.tensor([P], dtype=torch.int32, device=dev)
+            t_l = _time(lambda: ops.paged_attn_prefill(qc, kc, vct, bt[:1], cu, ctx, P, H, G, d, d ** -0.5, out=o), 5)
+            keys_b = sum(i % chunk + 1 for i in range(P))
+            row("softmax_bias_attn (value-less term, head gates)", f"prefill {P} tokens, chunks of {chunk}, {H}/{G} heads x {d}", t_n,
+                "mfma", 2.0 * keys_b * H * 2 * d, "paged_attn_prefill (causal softmax)", t_l, 2.0 * (P * (P + 1) // 2) * H * 2 * d)
+        else:
+            ctxd = torch.full((batch,), P, dtype=torch.int32, device=dev)
+            ws = torch.empty(max(ops.decode_workspace_bytes(batch, H, d, 16), 16), dtype=torch.uint8, device=dev)
+            t_l = _time(lambda: ops.paged_attn_decode(qc, kc, vct, bt, ctxd, H, G, d, d ** -0.5, num_splits=4, workspace=ws, out=o))
+            kb = (P - 1) % chunk + 1
+            row("softmax_bias_attn (value-less term, head gates)", f"decode {T} rows at position {P - 1}: {kb} keys each, chunks of {chunk}",
+                t_n, "hbm", T * kb * G * 2 * d * 2, f"paged_attn_decode (whole context: {P} keys each)", t_l, T * P * G * 2 * d * 2)
+    # ---- the mixture (choice by logits, softmax over the chosen, biased router; the shared expert's rows come
+    # ---- from the layer's output product) beside the Tafisun design's (softmax route in groups, identity and
+    # ---- shared experts)
+    E, top, Fe = 32, 4, W // 2
+    lw = SimpleNamespace(router_w=rnd(E, W, dt=torch.float32) * W ** -0.5, router_b=torch.zeros(E, device=dev),
+                         correction=torch.zeros(E, device=dev), gate_up_w=rnd(E, 2 * Fe, W) * W ** -0.5,
+                         down_w=rnd(E, W, Fe) * Fe ** -0.5)
+    ff = MoEFeedForward(MoESpec(E, top, 1, 1, Fe, score="chosen_softmax", router_bias=True, shared_gated=False), lw, None)
+    lin = SimpleNamespace(linear=lambda x, w: ops.linear_decode(x, w) if x.shape[0] <= ops.LINEAR_DECODE_MAX_M else torch.mm(x, w.t()))
+    lw0 = SimpleNamespace(router_w=rnd(E + 1, W, dt=torch.float32) * W ** -0.5, correction=torch.zeros(E, device=dev),
+                          gate_up_w=rnd(E - 2, 2 * Fe, W) * W ** -0.5, down_w=rnd(E - 2, W, Fe) * Fe ** -0.5,
+                          shared_gate_up_w=rnd(2 * Fe, W) * W ** -0.5, shared_down_w=rnd(W, Fe) * Fe ** -0.5)
+    ff0 = MoEFeedForward(MoESpec(E - 2, top, 4, 2, Fe, score="softmax", group_score="max", weight_scale=1.5, identity=2, limit=7.0,
+                                 shared_ff=Fe, shared_limit=7.0), lw0, lin)
+    for T, tag in ((P, "prefill"), (batch, "decode")):
+        h, other = rnd(T, W), rnd(T, W)
+        t_n, t_l = _time(lambda: ff(h, shared=other), 5), _time(lambda: ff0(h), 5)
+        if tag == "prefill":
+            row("mixture (choice by logits, softmax over the chosen)", f"prefill {T} rows, {top} of {E} x {Fe}", t_n, "mfma",
+                6.0 * T * top * Fe * W, "mixture (softmax route in groups, identity, limits, shared expert)", t_l,
+                6.0 * T * (top + 1) * Fe * W)
+        else:
+            row("mixture (choice by logits, softmax over the chosen)", f"decode {T} rows, {top} of {E} x {Fe}", t_n, "hbm",
+                min(E, T * top) * 3 * Fe * W * 2, "mixture (softmax route in groups, identity, limits, shared expert)", t_l,
+                (min(E - 2, T * top) + 1) * 3 * Fe * W * 2)
+    return rows
+
+
+def compare_bemulorn(widths, layers: int, batch: int, prompt_len: int, steps: int, warmup: int) -> dict:
+    """The Bemulorn design beside the closest existing model, a Llama-shaped decoder (rotary
+    grouped-query softmax attention, gated feed-forward) of equal width, depth and weights per layer."""
+    result = {"metric": "bemulorn_vs_llama_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+              "config": {"layers": layers, "batch": batch, "prompt_len": prompt_len, "decode_steps": steps},
+              "models": [], "kernels": {}}
+    for width in widths:
+        bc = ModelConfig.from_dict(bemulorn_config(width, layers, max_positions=prompt_len + steps + warmup + 16))
+        b = through_engine(bc, batch, prompt_len, steps, warmup)
+        lc = ModelConfig.from_dict(llama_config(width, layers, b["params_per_layer"]))
+        ll = through_engine(lc, batch, prompt_len, steps, warmup)
+        result["models"].append({"width": width, "layers": layers, "bemulorn": b, "llama": ll,
+                                 "prefill_ratio": round(b["prefill_tok_s"] / ll["prefill_tok_s"], 3),
+                                 "decode_ratio": round(b["decode_tok_s"] / ll["decode_tok_s"], 3)})
+        result["kernels"][str(width)] = bemulorn_kernel_table(width, prompt_len, batch)
     return result

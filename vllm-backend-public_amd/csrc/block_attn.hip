@@ -20,6 +20,7 @@ namespace mi355 {
 
 constexpr int kPageB = MI355_BLOCK_SIZE;
 constexpr float kLog2eB = 1.4426950408889634f;
+constexpr float kLazyLog2 = 8.0f;
 
 // one workgroup per packed row, one wave per head in turn
 template <typename T>
@@ -298,17 +299,22 @@ __global__ __launch_bounds__(256) void softmax_bias_attn_mfma_kernel(
       }
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      // The reference of the exponentials follows the maximum only when that grew by more than kLazyLog2:
+      // below that the weights of this and later tiles reach 2^kLazyLog2 at most (harmless in fp32 sums and
+      // in the 16-bit A operand, whose relative precision does not depend on the magnitude), and the
+      // accumulators of all heads are spared a rescale in nearly every tile.
       const float mn = fmaxf(m[i], tmax);
-      corr[i] = __builtin_amdgcn_exp2f(m[i] - mn);
-      m[i] = mn;
+      const bool grow = mn - m[i] > kLazyLog2;
+      corr[i] = grow ? __builtin_amdgcn_exp2f(m[i] - mn) : 1.0f;
+      if (grow) m[i] = mn;
       l[i] *= corr[i];
-      moved |= corr[i] != 1.0f;
+      moved |= grow;
       float w[2][4];
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          w[half][r] = vis[half][r] ? __builtin_amdgcn_exp2f(sc[half][r] - mn) : 0.f;
+          w[half][r] = vis[half][r] ? __builtin_amdgcn_exp2f(sc[half][r] - m[i]) : 0.f;
           l[i] += w[half][r];
         }
       }

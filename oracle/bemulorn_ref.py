@@ -17,8 +17,8 @@ keys) and `vdim` (values) channels; q, k, v = Q h + bq, K h + bk, V h + bv.
     w_i <- w_i / s * m_i + w_i (1 - m_i), and cos, sin are both multiplied by 0.1 ln s + 1;
   * score_ij = q_i . k_j * scale; position i sees j <= i with i // size == j // size (mask.size;
     chunks count from position 0 of the sequence);
-  * weights p_ij = exp(s_ij) / (1 + sum_j exp(s_ij)): the denominator holds one more term whose
-    score is 0 and which carries no value;
+  * weights p_ij = exp(s_ij) / (1 + sum_j exp(s_ij)): the denominator is one larger than the sum over
+    the keys (an extra term exp(0) to which no value belongs);
   * head h's output is multiplied by sigmoid(g_h . h_in), then O on the concatenated heads;
   * "kv_from": j: the layer has no K, V of its own and attends to the rotated keys and the values
     that layer j computed for the same tokens.

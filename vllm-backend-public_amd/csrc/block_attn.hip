@@ -158,8 +158,8 @@ __global__ __launch_bounds__(64) void softmax_bias_attn_kernel(
 // are loaded once for the HB heads.  Keys go 32 at a time (two pages).  Scores are computed
 // transposed, S^T = K Q^T: a lane then holds, for its query (lane % 16), the scores of keys
 // 4 (lane / 16) + r of either page -- after the exponential exactly an A-operand fragment of P V, V
-// pages being [vdim, 16 tokens].  The softmax runs on line in base 2 (running maximum and sum per
-// query and head; accumulators are rescaled only when some maximum moved).  Rows of one tile may
+// pages being [vdim, 16 tokens].  The softmax runs on line in base 2 (a reference and a sum per query and
+// head; the reference follows the running maximum lazily, and accumulators are rescaled only then).  Rows of one tile may
 // lie in two blocks: the walk starts at the first row's block and every row masks for itself.
 // gridDim.z > 1: the 32-key tiles are dealt out to the z workgroups in turn, each leaves its
 // accumulators, maxima and sums in fp32 scratch, and bias_attn_merge_kernel joins them.

@@ -292,6 +292,21 @@ int32_t mi355_paged_attn_prefill(void* out, int64_t out_stride, const void* q,
                                  int32_t max_q_len, int32_t num_heads,
                                  int32_t num_kv_heads, int32_t head_dim,
                                  float scale, int32_t dtype, void* stream);
+/*
+ * The same launch for attention inside chunks of positions (no counterpart in the reference): a
+ * query at position p sees the keys j with (p / chunk) * chunk <= j <= p (chunk 0: all j <= p);
+ * sink (fp32 [num_heads], may be null): one more term exp(sink[h]) in the softmax denominator,
+ * without a value; gate (dtype, rows gate_stride apart, may be null): the output of (token, head) is
+ * multiplied by sigmoid(gate[token, head]).  Pages as above with v_dim == head_dim.
+ */
+int32_t mi355_paged_attn_prefill_ext(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                     const void* k_cache, const void* v_cache, int32_t num_blocks,
+                                     const int32_t* block_tables, int32_t max_blocks_per_seq,
+                                     const int32_t* cu_seqlens, const int32_t* context_lens,
+                                     int32_t num_seqs, int32_t max_q_len, int32_t num_heads,
+                                     int32_t num_kv_heads, int32_t head_dim, float scale,
+                                     int32_t chunk, const float* sink, const void* gate,
+                                     int64_t gate_stride, int32_t dtype, void* stream);
 
 /*
  * SwiGLU gate:  out[t, :] = round(round(silu(x[t, :F])) * x[t, F:2F]).

@@ -66,13 +66,13 @@ CONFIGS = {
                          {"type": "attention", "mixer": _attn(1, 1, 136, 40, 40, 0.1, _rot(64, 10000.0, 8.0, 32, 4.0, 1.0)),
                           "mlp": None},
                          {"type": "attention", "mixer": _attn(4, 1, 8, 12, 16, 0.5, _rot(8, 100.0), kv_from=1), "mlp": _dense(24, 7.0)}]},
-    # sizes that the matrix-core attention, the matrix-core expert rows and (width 512) the tiled weight
-    # stream cover in 16 bits
+    # sizes that the matrix-core attention (layers 0 and 1 also its LDS-staged form for prompts: equal key and
+    # value sizes of 64), the matrix-core expert rows and (width 512) the tiled weight stream cover in 16 bits
     "wide": {"architecture": "Bemulorn", "width": 512, "vocab": 384, "max_positions": 320, "norm": {"eps": 1e-6},
              "embedding": {"scale": 2.0}, "logit_scale": 1.5,
-             "layers": [{"type": "attention", "mixer": _attn(8, 2, 64, 32, 48, 0.125, _rot(32, 10000.0, 4.0, 128, 32.0, 1.0)),
+             "layers": [{"type": "attention", "mixer": _attn(8, 2, 64, 64, 48, 0.125, _rot(32, 10000.0, 4.0, 128, 32.0, 1.0)),
                          "mlp": _moe(8, 2, 256, shared=128)},
-                        {"type": "attention", "mixer": _attn(6, 2, 64, 32, 33, 0.1, _rot(32, 10000.0, 4.0, 128, 32.0, 1.0), kv_from=0),
+                        {"type": "attention", "mixer": _attn(6, 2, 64, 64, 33, 0.1, _rot(32, 10000.0, 4.0, 128, 32.0, 1.0), kv_from=0),
                          "mlp": _dense(1024, 1.5)},
                         {"type": "attention", "mixer": _attn(6, 2, 32, 48, 0, 0.2, _rot(16, 1000.0)), "mlp": _moe(16, 4, 128)}]},
     # a width that is no multiple of 8, head and expert sizes that no matrix-core tile covers, five
@@ -188,7 +188,7 @@ def _pages(T, G, d, dv, dtype, spare=3, seed=0):
     return kc, vc, bt, slots
 
 
-def _attend_in_cuts(q, k, v, gate, cuts, size, scale, rot=None, tiled=False, splits=0, sink=True):
+def _attend_in_cuts(q, k, v, gate, cuts, size, scale, rot=None, tiled=False, splits=0, sink=True, staged=False):
     """q [T, H, d], k [T, G, d], v [T, G, dv] unrotated, gate [T, H]: rotation + page write + attention
     through the product's kernels, portion by portion, over shuffled NaN-filled pages; the output lands in
     a column slice of a wider NaN-filled row."""
@@ -215,11 +215,18 @@ def _attend_in_cuts(q, k, v, gate, cuts, size, scale, rot=None, tiled=False, spl
         vs, gs = buf[:, (H + G) * d: (H + G) * d + G * dv], buf[:, (H + G) * d + G * dv: width]
         ops.rope_partial_kv_write(qs, ks, vs, table, pos, slots[at:at + n], kc, vc, H, G, d, dv)
         tiles = torch.from_numpy(ops.query_tiles(np.array([0, n]))).cuda() if tiled else None
-        row = torch.full((n, H * dv + 11), float("nan"), dtype=dt, device="cuda")
-        ops.softmax_bias_attn(qs, kc, vc, bt, torch.zeros(n, dtype=torch.int32, device="cuda"), pos, None, None, gs, H, scale,
-                              block=size, tiles=tiles, num_splits=splits, sink=sink_t, out=row[:, 3: 3 + H * dv])
-        assert torch.isnan(row[:, :3]).all() and torch.isnan(row[:, 3 + H * dv:]).all()
-        outs.append(row[:, 3: 3 + H * dv].float().cpu())
+        lead = 8 if staged else 3                                # (the staged form wants 16-byte aligned rows)
+        row = torch.full((n, H * dv + 16), float("nan"), dtype=dt, device="cuda")
+        if staged:
+            assert ops.chunk_attn_prefill_ok(dt, H, G, d, dv)
+            ops.paged_attn_prefill_ext(qs, kc, vc, bt, torch.tensor([0, n], dtype=torch.int32, device="cuda"),
+                                       torch.tensor([at + n], dtype=torch.int32, device="cuda"), n, H, G, d, scale, chunk=size,
+                                       sink=sink_t, gate=gs, out=row[:, lead: lead + H * dv])
+        else:
+            ops.softmax_bias_attn(qs, kc, vc, bt, torch.zeros(n, dtype=torch.int32, device="cuda"), pos, None, None, gs, H, scale,
+                                  block=size, tiles=tiles, num_splits=splits, sink=sink_t, out=row[:, lead: lead + H * dv])
+        assert torch.isnan(row[:, :lead]).all() and torch.isnan(row[:, lead + H * dv:]).all()
+        outs.append(row[:, lead: lead + H * dv].float().cpu())
         at += n
     return torch.cat(outs)
 
@@ -272,6 +279,26 @@ def test_attention_on_the_matrix_cores(H, G, d, dv, size, rot):
             assert (got - ref).abs().max() <= 3e-2 * ref.abs().max(), (cuts, sink)
 
 
+@pytest.mark.parametrize("T", [75, 300])
+@pytest.mark.parametrize("H,G,d,size,rot", [(8, 2, 64, 48, _rot(32, 10000.0, 4.0, 128, 32.0, 1.0)), (4, 4, 64, 7, _RB), (16, 4, 128, 20, _RA),
+                                            (6, 1, 128, 0, _rot(64, 10000.0)), (3, 1, 64, 33, None), (16, 1, 64, 100, _rot(64, 100.0)),
+                                            (2, 2, 128, 1, None), (12, 3, 128, 64, _rot(32, 500000.0)), (5, 1, 64, 128, _RA)])
+def test_attention_staged_through_lds(H, G, d, size, rot, T):
+    """The form for prompts and portions (equal key and value sizes of 64 or 128, bfloat16): K/V steps staged
+    through LDS for a workgroup's tile of queries.  Chunks that end inside a step, a tile and a page; walks
+    that start several steps into the sequence; portions that begin and end anywhere; with and without the
+    value-less term."""
+    g = torch.Generator().manual_seed(H * 100 + d + T)
+    b16 = lambda t: t.to(torch.bfloat16)                      # noqa: E731
+    q, k, v = b16(torch.randn(T, H, d, generator=g)), b16(torch.randn(T, G, d, generator=g)), b16(torch.randn(T, G, d, generator=g))
+    gate = b16(torch.randn(T, H, generator=g) * 2)
+    for sink in (True, False):
+        ref = _attend_ref(q.float(), k.float(), v.float(), gate.float(), size, 0.3, rot, sink=sink)
+        for cuts in ([T], [2, 3, 1, 30, 2, 16, 21], [T // 2 + 3, 1, 1, 2]) + (([1] * T,) if T == 75 and sink else ()):
+            got = _attend_in_cuts(q, k, v, gate, cuts, size, 0.3, rot, staged=True, sink=sink)
+            assert (got - ref).abs().max() <= 3e-2 * ref.abs().max(), (cuts, sink)
+
+
 @pytest.mark.parametrize("size", [16, 17, 31, 48, 64, 65, 400])
 def test_chunk_edge_shows_with_one_loud_key(size):
     """The first token of the second chunk holds a key that every query scores far above all others
@@ -300,6 +327,14 @@ def test_chunk_edge_shows_with_one_loud_key(size):
         b16 = lambda t: t.to(torch.bfloat16)                  # noqa: E731
         got = _attend_in_cuts(b16(q), b16(k), b16(v), b16(gate), cuts, size, 1.0, rot, tiled=True, splits=4)
         r16 = _attend_ref(b16(q).float(), b16(k).float(), b16(v).float(), b16(gate).float(), size, 1.0, rot)
+        assert (got - r16).abs().max() <= 3e-2 * r16.abs().max(), cuts
+    # the same key through the LDS-staged form (equal key and value sizes of 64): pad both with silent channels
+    q6, k6, v6 = torch.zeros(T, H, 64), torch.zeros(T, G, 64), torch.zeros(T, G, 64)
+    q6[..., :d], k6[..., :d], v6[..., :dv] = q, k, v
+    r16 = _attend_ref(b16(q6).float(), b16(k6).float(), b16(v6).float(), b16(gate).float(), size, 1.0, rot)
+    assert float(r16[last_in, 5]) > 4.9 and abs(float(r16[first_out, 5])) < 1e-3
+    for cuts in ([T], [last_in, 1, 1], [5, 2, j0 - 7, 1, 2, 2], [j0 + 1, size - 2, 1, 1]):
+        got = _attend_in_cuts(b16(q6), b16(k6), b16(v6), b16(gate), cuts, size, 1.0, rot, staged=True)
         assert (got - r16).abs().max() <= 3e-2 * r16.abs().max(), cuts
 
 

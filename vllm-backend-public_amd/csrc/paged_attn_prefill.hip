@@ -28,6 +28,12 @@
 // rows as the A operand, and O^T += V^T . P^T with the transposed V page as the A operand
 // and the lane's own probabilities as B.  The causal mask is applied per column (key <=
 // position of the column's query).
+//
+// EXT (a second set of instantiations; the plain ones compile as before): attention inside chunks of
+// positions -- a column at position p sees the keys from (p / chunk) * chunk on, the walk starts at the
+// chunk of the tile's first query and columns of a tile that straddles a chunk edge mask for themselves;
+// one more term exp(sink[head]) in the softmax denominator that carries no value; and the output times
+// the sigmoid of one gate number per (token, head).
 #include "common.h"
 
 #include <math.h>
@@ -48,12 +54,13 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
 
 // Second launch bound: waves per SIMD the register allocation must leave room for.  Two workgroups
 // per CU overlap each other's dependent chains (LDS reads -> MFMAs -> exp2 -> MFMAs -> barrier).
-template <typename T, int D, int NQ>
+template <typename T, int D, int NQ, bool EXT>
 __global__ __launch_bounds__(kPrefillThreads, NQ <= 2 ? 2 : 1) void paged_attn_prefill_kernel(
     uint16_t* __restrict__ out, int64_t out_stride, const uint16_t* __restrict__ q, int64_t q_stride,
     const uint16_t* __restrict__ k_cache, const uint16_t* __restrict__ v_cache, int num_blocks,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ cu_seqlens,
-    const int32_t* __restrict__ context_lens, int num_heads, int num_kv_heads, float scale_log2e, int qt) {
+    const int32_t* __restrict__ context_lens, int num_heads, int num_kv_heads, float scale_log2e, int qt,
+    int chunk, const float* __restrict__ sink, const uint16_t* __restrict__ gate, int64_t gate_stride) {
   constexpr int KS = D / 32;
   constexpr int NT = D / 16;
   constexpr int BS = MI355_BLOCK_SIZE;
@@ -104,7 +111,7 @@ __global__ __launch_bounds__(kPrefillThreads, NQ <= 2 ? 2 : 1) void paged_attn_p
   if (pos0 < 0) return;                          // inconsistent lengths: nothing sensible to compute
 
   // this lane's columns: pair index p = (wave*NQ + t)*16 + c -> (query, head)
-  int col_q[NQ], col_head[NQ], col_pos[NQ];
+  int col_q[NQ], col_head[NQ], col_pos[NQ], col_lo[NQ];
   bool col_ok[NQ];
   uint4 qf[NQ][KS];                              // the lane's query fragments (B operands), read once
 #pragma unroll
@@ -114,6 +121,7 @@ __global__ __launch_bounds__(kPrefillThreads, NQ <= 2 ? 2 : 1) void paged_attn_p
     col_head[t] = kvh * group + p % group;
     col_ok[t] = (p < qt * group) && (col_q[t] < q_len);
     col_pos[t] = col_ok[t] ? pos0 + col_q[t] : -1;
+    col_lo[t] = (EXT && chunk > 0 && col_ok[t]) ? (col_pos[t] / chunk) * chunk : 0;      // first key the column sees
     const uint16_t* qp = q + (q_begin + (col_ok[t] ? col_q[t] : 0)) * q_stride +
                          static_cast<int64_t>(col_ok[t] ? col_head[t] : 0) * D + 8 * h;
 #pragma unroll
@@ -128,6 +136,16 @@ __global__ __launch_bounds__(kPrefillThreads, NQ <= 2 ? 2 : 1) void paged_attn_p
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) kmin = min(kmin, __shfl_xor(kmin, off, 64));
   const int t_min = __builtin_amdgcn_readfirstlane(kmin);
+  int lomax = 0;                                                  // largest first-visible key among the wave's columns
+  if (EXT) {
+#pragma unroll
+    for (int t = 0; t < NQ; ++t) lomax = max(lomax, col_lo[t]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) lomax = max(lomax, __shfl_xor(lomax, off, 64));
+  }
+  const int t_lo_max = __builtin_amdgcn_readfirstlane(lomax);
+  // the walk starts at the chunk of the tile's first query, on a boundary of the barrier interval (HS steps)
+  const int s0 = (EXT && chunk > 0) ? ((pos0 + q0) / chunk) * chunk / 64 * 2 : 0;
   const int t_end_wg = pos0 + min(q0 + qt, q_len);              // the tile's last query sees keys [0, t_end_wg)
 
   const int32_t* bt = block_tables + static_cast<int64_t>(seq) * max_blocks;
@@ -229,6 +247,16 @@ __global__ __launch_bounds__(kPrefillThreads, NQ <= 2 ? 2 : 1) void paged_attn_p
         }
       }
     }
+    if (EXT && s * 32 < t_lo_max) {        // wave-uniform: ahead of the chunk of some column
+#pragma unroll
+      for (int t = 0; t < NQ; ++t) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          sa[t][j] = (tok0 + j >= col_lo[t]) ? sa[t][j] : -INFINITY;
+          sb[t][j] = (tok0 + 4 + j >= col_lo[t]) ? sb[t][j] : -INFINITY;
+        }
+      }
+    }
   };
 
   // ================= one pass: scores, probabilities against a lazy reference, O =================
@@ -315,14 +343,14 @@ __global__ __launch_bounds__(kPrefillThreads, NQ <= 2 ? 2 : 1) void paged_attn_p
 #pragma unroll
     for (int hs = 0; hs < HS; ++hs) {          // images beyond the last step re-read the last pages (clamped), unused
       pvec r0[PPT];
-      stage_load(r0, hs * 32);
-      stage_store(r0, hs, hs * 32);
+      stage_load(r0, (s0 + hs) * 32);
+      stage_store(r0, hs, (s0 + hs) * 32);
     }
   }
   __syncthreads();
-  for (int s = 0; s < steps; s += HS) {
+  for (int s = s0; s < steps; s += HS) {
     const bool more = s + HS < steps;
-    const int par = (s / HS) & 1;
+    const int par = ((s - s0) / HS) & 1;
     pvec nxt[HS][PPT];
     if (more) {                                                  // workgroup-uniform branch
 #pragma unroll
@@ -344,7 +372,11 @@ __global__ __launch_bounds__(kPrefillThreads, NQ <= 2 ? 2 : 1) void paged_attn_p
     lt += __shfl_xor(lt, 16, 64);
     lt += __shfl_xor(lt, 32, 64);
     if (!col_ok[t]) continue;
-    const float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    if (EXT && sink != nullptr)          // the value-less term, against the column's reference (a valid column has seen a key)
+      lt += __builtin_amdgcn_exp2f(MI355_LD(float, sink, sink + col_head[t]) * 1.4426950408889634f - m_ref[t]);
+    float inv = lt > 0.f ? 1.0f / lt : 0.f;
+    if (EXT && gate != nullptr)
+      inv /= 1.0f + expf(-T::to_f(MI355_LD(uint16_t, gate, gate + (q_begin + col_q[t]) * gate_stride + col_head[t])));
     uint16_t* op = out + (q_begin + col_q[t]) * out_stride + static_cast<int64_t>(col_head[t]) * D + 4 * h;
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
@@ -360,7 +392,8 @@ __global__ __launch_bounds__(kPrefillThreads, NQ <= 2 ? 2 : 1) void paged_attn_p
 
 }  // namespace mi355
 
-extern "C" int32_t mi355_paged_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+static int32_t launch_paged_attn_prefill(const char* name, bool ext, int32_t chunk, const float* sink, const void* gate,
+                                          int64_t gate_stride, void* out, int64_t out_stride, const void* q, int64_t q_stride,
                                             const void* k_cache, const void* v_cache, int32_t num_blocks,
                                             const int32_t* block_tables, int32_t max_blocks_per_seq,
                                             const int32_t* cu_seqlens, const int32_t* context_lens,
@@ -368,7 +401,6 @@ extern "C" int32_t mi355_paged_attn_prefill(void* out, int64_t out_stride, const
                                             int32_t num_kv_heads, int32_t head_dim, float scale,
                                             int32_t dtype, void* stream) {
   using namespace mi355;
-  const char* name = "mi355_paged_attn_prefill";
   MI355_REQUIRE(out && q && k_cache && v_cache && block_tables && cu_seqlens && context_lens,
                 MI355_ERR_INVALID, "%s: null pointer", name);
   MI355_REQUIRE(num_seqs >= 0 && num_seqs <= 65535 && num_blocks > 0 && max_blocks_per_seq > 0 &&
@@ -403,12 +435,18 @@ extern "C" int32_t mi355_paged_attn_prefill(void* out, int64_t out_stride, const
   const int qt = 64 * nq / group;                      // queries per workgroup (>= 4: group <= 16)
   dim3 grid((max_q_len + qt - 1) / qt, num_kv_heads, num_seqs), block(kPrefillThreads);
   hipStream_t s = static_cast<hipStream_t>(stream);
-#define MI355_PRE(TT, DD, NN)                                                                           \
-  hipLaunchKernelGGL((paged_attn_prefill_kernel<TT, DD, NN>), grid, block, 0, s,                        \
+#define MI355_PRE_E(TT, DD, NN, EE)                                                                     \
+  hipLaunchKernelGGL((paged_attn_prefill_kernel<TT, DD, NN, EE>), grid, block, 0, s,                    \
                      static_cast<uint16_t*>(out), out_stride, static_cast<const uint16_t*>(q), q_stride, \
                      static_cast<const uint16_t*>(k_cache), static_cast<const uint16_t*>(v_cache),      \
                      num_blocks, block_tables, max_blocks_per_seq, cu_seqlens, context_lens, num_heads, \
-                     num_kv_heads, scale * 1.4426950408889634f, qt)
+                     num_kv_heads, scale * 1.4426950408889634f, qt, chunk, sink,                        \
+                     static_cast<const uint16_t*>(gate), gate_stride)
+#define MI355_PRE(TT, DD, NN)                                                                           \
+  do {                                                                                                  \
+    if (ext) MI355_PRE_E(TT, DD, NN, true);                                                             \
+    else MI355_PRE_E(TT, DD, NN, false);                                                                \
+  } while (0)
 #define MI355_PRE_NQ(TT, DD)                \
   switch (nq) {                             \
     case 1: MI355_PRE(TT, DD, 1); break;    \
@@ -421,5 +459,33 @@ extern "C" int32_t mi355_paged_attn_prefill(void* out, int64_t out_stride, const
   }
 #undef MI355_PRE_NQ
 #undef MI355_PRE
+#undef MI355_PRE_E
   return check_launch(name);
+}
+
+extern "C" int32_t mi355_paged_attn_prefill(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                            const void* k_cache, const void* v_cache, int32_t num_blocks,
+                                            const int32_t* block_tables, int32_t max_blocks_per_seq,
+                                            const int32_t* cu_seqlens, const int32_t* context_lens,
+                                            int32_t num_seqs, int32_t max_q_len, int32_t num_heads,
+                                            int32_t num_kv_heads, int32_t head_dim, float scale,
+                                            int32_t dtype, void* stream) {
+  return launch_paged_attn_prefill("mi355_paged_attn_prefill", false, 0, nullptr, nullptr, 0, out, out_stride, q, q_stride, k_cache,
+                                   v_cache, num_blocks, block_tables, max_blocks_per_seq, cu_seqlens, context_lens, num_seqs,
+                                   max_q_len, num_heads, num_kv_heads, head_dim, scale, dtype, stream);
+}
+
+extern "C" int32_t mi355_paged_attn_prefill_ext(void* out, int64_t out_stride, const void* q, int64_t q_stride,
+                                                const void* k_cache, const void* v_cache, int32_t num_blocks,
+                                                const int32_t* block_tables, int32_t max_blocks_per_seq,
+                                                const int32_t* cu_seqlens, const int32_t* context_lens,
+                                                int32_t num_seqs, int32_t max_q_len, int32_t num_heads,
+                                                int32_t num_kv_heads, int32_t head_dim, float scale, int32_t chunk,
+                                                const float* sink, const void* gate, int64_t gate_stride,
+                                                int32_t dtype, void* stream) {
+  MI355_REQUIRE(chunk >= 0 && (gate == nullptr || gate_stride >= num_heads), MI355_ERR_INVALID,
+                "mi355_paged_attn_prefill_ext: chunk %d, gate rows shorter than the heads", chunk);
+  return launch_paged_attn_prefill("mi355_paged_attn_prefill_ext", true, chunk, sink, gate, gate_stride, out, out_stride, q,
+                                   q_stride, k_cache, v_cache, num_blocks, block_tables, max_blocks_per_seq, cu_seqlens,
+                                   context_lens, num_seqs, max_q_len, num_heads, num_kv_heads, head_dim, scale, dtype, stream);
 }

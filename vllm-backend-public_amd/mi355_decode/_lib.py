@@ -50,6 +50,8 @@ def _load() -> ctypes.CDLL:
         "mi355_paged_attn_decode_static": (I32, [P, P, I64, P, P, I32, P, I32, P, I32, I32, I32, I32, F, I32, I32, P]),
         "mi355_paged_attn_prefill": (I32, [P, I64, P, I64, P, P, I32, P, I32, P, P, I32, I32, I32, I32, I32,
                                            F, I32, P]),
+        "mi355_paged_attn_prefill_ext": (I32, [P, I64, P, I64, P, P, I32, P, I32, P, P, I32, I32, I32, I32, I32,
+                                               F, I32, P, P, I64, I32, P]),
         "mi355_silu_and_mul": (I32, [P, P, I64, I64, I32, I32, P]),
         "mi355_sum_slabs": (I32, [P, I64, P, I32, P, I32, I32, I32, P]),
         "mi355_silu_and_mul_slabs": (I32, [P, I64, P, I32, I32, I32, I32, P]),
@@ -157,7 +159,7 @@ lib = _load()
 EXPORTS = ("mi355_abi_version", "mi355_last_error", "mi355_target_arch",
            "mi355_bounds_enabled", "mi355_bounds_set_ranges", "mi355_bounds_report", "mi355_rms_norm",
            "mi355_fused_add_rms_norm", "mi355_rope_kv_write", "mi355_paged_attn_decode_workspace",
-           "mi355_paged_attn_decode", "mi355_paged_attn_decode_static", "mi355_paged_attn_prefill", "mi355_silu_and_mul", "mi355_sum_slabs", "mi355_silu_and_mul_slabs", "mi355_argmax",
+           "mi355_paged_attn_decode", "mi355_paged_attn_decode_static", "mi355_paged_attn_prefill", "mi355_paged_attn_prefill_ext", "mi355_silu_and_mul", "mi355_sum_slabs", "mi355_silu_and_mul_slabs", "mi355_argmax",
            "mi355_argmax_chunked", "mi355_embed_rms_norm",
            "mi355_layer_norm", "mi355_fused_add_layer_norm", "mi355_embed_pos_layer_norm", "mi355_relu",
            "mi355_argmax_shard_key", "mi355_argmax_key_to_index",

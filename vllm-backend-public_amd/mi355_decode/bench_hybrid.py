@@ -668,7 +668,12 @@ def bemulorn_kernel_table(width: int, prompt_len: int, batch: int) -> list:
             cu, ctx = torch.tensor([0, P], dtype=torch.int32, device=dev), torch.tensor([P], dtype=torch.int32, device=dev)
             t_l = _time(lambda: ops.paged_attn_prefill(qc, kc, vct, bt[:1], cu, ctx, P, H, G, d, d ** -0.5, out=o), 5)
             keys_b = sum(i % chunk + 1 for i in range(P))
-            row("softmax_bias_attn (value-less term, head gates)", f"prefill {P} tokens, chunks of {chunk}, {H}/{G} heads x {d}", t_n,
+            # what the runner takes for prompts at these sizes: the LDS-staged form
+            t_s = _time(lambda: ops.paged_attn_prefill_ext(q, kc, vct, bt[:1], cu, ctx, P, H, G, d, d ** -0.5, chunk=chunk, sink=sink,
+                                                           gate=gh, out=out_slice), 5)
+            row("paged_attn_prefill_ext (chunks, value-less term, head gates)", f"prefill {P} tokens, chunks of {chunk}, {H}/{G} heads x {d}",
+                t_s, "mfma", 2.0 * keys_b * H * 2 * d, "paged_attn_prefill (causal softmax)", t_l, 2.0 * (P * (P + 1) // 2) * H * 2 * d)
+            row("softmax_bias_attn, tile form (prompts of other head sizes)", f"prefill {P} tokens, chunks of {chunk}, {H}/{G} heads x {d}", t_n,
                 "mfma", 2.0 * keys_b * H * 2 * d, "paged_attn_prefill (causal softmax)", t_l, 2.0 * (P * (P + 1) // 2) * H * 2 * d)
         else:
             ctxd = torch.full((batch,), P, dtype=torch.int32, device=dev)

@@ -67,10 +67,13 @@ def rotary_table(rot_dims: int, base: float, max_pos: int, device, scaling=None)
 class StepBatch:
     """Device-side description of one packed step (see csrc/seqmix.hip)."""
     __slots__ = ("ids", "positions", "slot_mapping", "block_tables", "cu_seqlens", "tok_seq", "state_slots",
-                 "num_tokens", "num_seqs", "tiles", "long_chunks", "pair_tiles")
+                 "num_tokens", "num_seqs", "tiles", "long_chunks", "pair_tiles", "context_lens", "max_q_len")
 
     def __init__(self, ids, positions, slot_mapping, block_tables, cu_seqlens, tok_seq, state_slots, tiles=None,
-                 long_chunks=False, pair_tiles=None):
+                 long_chunks=False, pair_tiles=None, context_lens=None, max_q_len=0):
+        # every chunk's length of context after the step (int32, on the device) and the longest chunk: what the
+        # LDS-staged prompt attention walks by; None: not known to this step (captured decode steps)
+        self.context_lens, self.max_q_len = context_lens, int(max_q_len)
         self.tiles = tiles                            # 16-row query tiles (ops.query_tiles) or None: one wave per row
         self.pair_tiles = pair_tiles                  # heads -> tiles of 16 (row, head) pairs (ops.pair_tiles), or None
         self.long_chunks = long_chunks                # some chunk holds several tokens (prompts and portions)
@@ -219,6 +222,12 @@ class RotaryBlockAttention:
         elif s.rot_dims > 0:
             ops.rope_partial_kv_write(q, None, None, table, b.positions, b.slot_mapping, None, None, s.heads, s.kv_heads,
                                       s.dim, s.vdim)
+        if b.long_chunks and b.context_lens is not None and ops.chunk_attn_prefill_ok(q.dtype, s.heads, s.kv_heads, s.dim, s.vdim) \
+                and proj.stride(0) % 8 == 0 and out.stride(0) % 8 == 0:
+            # prompts and portions (single tokens beside them ride along): K/V steps staged through LDS once for a
+            # workgroup's tile of queries
+            return ops.paged_attn_prefill_ext(q, kc, vc, b.block_tables, b.cu_seqlens, b.context_lens, b.max_q_len, s.heads,
+                                              s.kv_heads, s.dim, s.scale, chunk=s.block, sink=lw.sink, gate=col("g"), out=out)
         return ops.softmax_bias_attn(q, kc, vc, b.block_tables, b.tok_seq, b.positions, None, None, col("g"), s.heads, s.scale,
                                      block=s.block, tiles=b.tiles, num_splits=r.block_key_splits(b, s), sink=lw.sink, out=out)
 
@@ -731,7 +740,8 @@ class HybridRunner(ModelRunner):
         dev = self.device
         t = lambda a, dt: torch.from_numpy(np.ascontiguousarray(a)).to(dev, dtype=dt, non_blocking=True)  # noqa: E731
         resid = self._run_chunks(t(token_ids, torch.int64), t(positions, torch.int64), t(slot_mapping, torch.int64),
-                                 t(block_tables, torch.int32), t(cu_seqlens, torch.int32))
+                                 t(block_tables, torch.int32), t(cu_seqlens, torch.int32), t(context_lens, torch.int32),
+                                 max_q_len)
         rows = np.asarray(logit_rows, dtype=np.int64)
         if rows.size == 0:
             torch.cuda.current_stream().synchronize()
@@ -739,7 +749,8 @@ class HybridRunner(ModelRunner):
         z = self._logits(resid.index_select(0, t(rows, torch.int64)))
         return z.float().cpu().numpy()
 
-    def _run_chunks(self, token_ids, positions, slot_mapping, block_tables, cu_seqlens) -> torch.Tensor:
+    def _run_chunks(self, token_ids, positions, slot_mapping, block_tables, cu_seqlens, context_lens=None,
+                    max_q_len: int = 0) -> torch.Tensor:
         S = cu_seqlens.numel() - 1
         lens = (cu_seqlens[1:] - cu_seqlens[:-1]).to(torch.int64)
         tok_seq = torch.repeat_interleave(torch.arange(S, dtype=torch.int32, device=self.device), lens,
@@ -747,13 +758,15 @@ class HybridRunner(ModelRunner):
         slots = torch.from_numpy(self._step_state_slots).to(self.device, non_blocking=True)
         tiles = torch.from_numpy(self._step_tiles).to(self.device, non_blocking=True)
         return self._forward(StepBatch(token_ids, positions, slot_mapping, block_tables.contiguous(), cu_seqlens,
-                                       tok_seq, slots, tiles, self._step_long, pair_tiles=self._chunk_pair_tiles))
+                                       tok_seq, slots, tiles, self._step_long, pair_tiles=self._chunk_pair_tiles,
+                                       context_lens=None if context_lens is None else context_lens.to(torch.int32).contiguous(),
+                                       max_q_len=max_q_len))
 
     def prefill(self, token_ids: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor,
                 block_tables: torch.Tensor, cu_seqlens: torch.Tensor, context_lens: torch.Tensor,
                 max_q_len: int, want_logits: bool = True, score=None):
         """As ModelRunner.prefill: packed prompts (or prompt chunks), eager."""
-        resid = self._run_chunks(token_ids, positions, slot_mapping, block_tables, cu_seqlens)
+        resid = self._run_chunks(token_ids, positions, slot_mapping, block_tables, cu_seqlens, context_lens, max_q_len)
         if score is not None:
             k, srows, targets = score
             parts = []

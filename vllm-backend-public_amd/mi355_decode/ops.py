@@ -288,6 +288,42 @@ def paged_attn_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Te
     return out
 
 
+def chunk_attn_prefill_ok(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int, v_dim: int) -> bool:
+    """Whether paged_attn_prefill_ext covers these sizes (16-bit storage, equal key and value sizes of 64 or 128,
+    at most 16 query heads to a kv head)."""
+    return dtype in (torch.bfloat16, torch.float16) and head_dim == v_dim and head_dim in (64, 128) \
+        and num_heads % num_kv_heads == 0 and num_heads // num_kv_heads <= 16
+
+
+def paged_attn_prefill_ext(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                           cu_seqlens: torch.Tensor, context_lens: torch.Tensor, max_q_len: int, num_heads: int,
+                           num_kv_heads: int, head_dim: int, scale: float, chunk: int = 0, sink: torch.Tensor | None = None,
+                           gate: torch.Tensor | None = None, out: torch.Tensor | None = None):
+    """paged_attn_prefill (K/V steps staged through LDS for a workgroup's query tile) for attention inside
+    chunks of `chunk` positions counted from position 0 (0: plain causal), with one more value-less term
+    exp(sink[h]) in the softmax denominator (float32 [heads]) and the output times sigmoid(gate[t, h])
+    (gate [tokens, heads], a column slice is fine).  q and out may be column slices on 16-byte boundaries."""
+    dt = _dt16(q, "q")
+    T = q.shape[0]
+    nb = _check_cache(q, k_cache, v_cache, block_tables, num_kv_heads, head_dim)
+    S = block_tables.shape[0]
+    for t, n, cnt in ((cu_seqlens, "cu_seqlens", S + 1), (context_lens, "context_lens", S)):
+        _dev(t, n)
+        if t.dtype != torch.int32 or t.numel() != cnt or not t.is_contiguous():
+            raise ValueError(f"{n} must be contiguous int32 [{cnt}]")
+    if out is None:
+        out = torch.empty((T, num_heads * head_dim), dtype=q.dtype, device=q.device)
+    if out.dtype != q.dtype or tuple(out.shape) != (T, num_heads * head_dim):
+        raise ValueError("out must be [tokens, heads * head_dim] in the dtype of q")
+    check(lib.mi355_paged_attn_prefill_ext(
+        out.data_ptr(), _rows(out, "out"), q.data_ptr(), _cols(q, "q", num_heads * head_dim), k_cache.data_ptr(),
+        v_cache.data_ptr(), nb, block_tables.data_ptr(), block_tables.shape[1], cu_seqlens.data_ptr(), context_lens.data_ptr(),
+        S, int(max_q_len), num_heads, num_kv_heads, head_dim, float(scale), int(chunk),
+        None if sink is None else _f32(sink, "sink", num_heads), None if gate is None else _same(gate, q, "gate"),
+        0 if gate is None else _cols(gate, "gate", num_heads), dt, _stream()))
+    return out
+
+
 def silu_and_mul(x: torch.Tensor, out: torch.Tensor | None = None):
     dt = _dt16(x, "x")
     T, two_f = x.shape

@@ -205,7 +205,8 @@ class RotaryBlockAttention:
     (it writes them first) or those of the layer it shares with: biased projections, rotary positions
     on the first rot_dims coordinates of every head, one more value-less term in the softmax
     denominator, one sigmoid gate per head.  Writes the gated heads into `out`, a column slice of
-    the row that the layer's output matrix multiplies."""
+    the row that the layer's output matrix multiplies.  Steps that hold a portion of a prompt take the
+    LDS-staged launch where the sizes allow (ops.chunk_attn_prefill_ok), all others the tile form."""
 
     def __init__(self, spec, lw, runner, cache_index: int, writes: bool):
         self.s, self.lw, self.r, self.ci, self.writes = spec, lw, runner, cache_index, writes
